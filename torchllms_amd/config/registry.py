@@ -18,6 +18,7 @@ from .llama import ConfigError, LlamaConfig, llama_model_spec
 from .spec import ModelSpec
 from .taluvik import ARCHITECTURE as TALUVIK, TaluvikConfig, taluvik_model_spec
 from .vobolorn import ARCHITECTURE as VOBOLORN, VobolornConfig, vobolorn_model_spec
+from .kepevik import ARCHITECTURE as KEPEVIK, KepevikConfig, kepevik_model_spec, kepevik_sizes_from_tensors
 
 
 @dataclass(frozen=True)
@@ -44,6 +45,10 @@ class ArchSpec:
     #: typed configuration -> the contents of a config.json that ``config_from_dict`` reads back
     #: (None: the configuration's own ``to_dict()``, or its fields if it is a dataclass)
     config_to_dict: Optional[Callable[[Any], Dict[str, Any]]] = None
+
+    #: (typed configuration, tensor name -> shape of the folder's tensors) -> typed configuration: for an
+    #: architecture some of whose sizes config.json leaves to the tensors' shapes (None: config.json says all)
+    sizes_from_tensors: Optional[Callable[[Any, Dict[str, tuple]], Any]] = None
 
     def config_json(self, config) -> Dict[str, Any]:
         """What a model folder's config.json holds for this configuration; it names this architecture."""
@@ -115,7 +120,16 @@ def load_config(folder) -> tuple:
     with open(path) as f:
         d = json.load(f)
     arch = get_architecture(architecture_name(d))
-    return arch, arch.config_from_dict(d)
+    config = arch.config_from_dict(d)
+    if arch.sizes_from_tensors is not None:
+        from ..weights.loader import safetensors_files, tensor_shapes
+
+        try:
+            safetensors_files(folder)
+        except FileNotFoundError:
+            return arch, config  # a folder with a configuration alone: the sizes stay as config.json and defaults give them
+        config = arch.sizes_from_tensors(config, tensor_shapes(folder))
+    return arch, config
 
 
 def _llama_rules(cfg: LlamaConfig):
@@ -185,5 +199,29 @@ register_architecture(
         weight_rules=_vobolorn_rules,
         stop_token_ids=_vobolorn_stop_ids,
         config_type=VobolornConfig,
+    )
+)
+
+
+def _kepevik_rules(cfg: KepevikConfig):
+    from ..weights.names import kepevik_name_rules
+
+    return kepevik_name_rules(cfg)
+
+
+def _kepevik_stop_ids(cfg: KepevikConfig):
+    eos = cfg.eos_token_id
+    return [] if eos is None else (list(eos) if isinstance(eos, (list, tuple)) else [eos])
+
+
+register_architecture(
+    ArchSpec(
+        name=KEPEVIK,
+        config_from_dict=KepevikConfig.from_dict,
+        model_spec=kepevik_model_spec,
+        weight_rules=_kepevik_rules,
+        stop_token_ids=_kepevik_stop_ids,
+        config_type=KepevikConfig,
+        sizes_from_tensors=kepevik_sizes_from_tensors,
     )
 )

@@ -516,7 +516,10 @@ __device__ __forceinline__ float row_group_sum(float v, int width) {
 
 // kDeltaRows: rows of a column that a lane holds (8 for keys of up to 128 channels, else 16; a column's lanes lie
 // in one row of 16 lanes).
-template <typename T, bool VEC, int kDeltaRows, int kDeltaCols>
+// CH: a decay of its own for every key channel (row of S) of a head: the pre-activations come as 32-bit rows
+// a_ch [n_tokens, a_stride] with H * dk columns, dt_bias has H * dk entries, and a token's decays lie in LDS beside
+// its key; the column a_off of proj is not read.
+template <typename T, bool VEC, int kDeltaRows, int kDeltaCols, bool CH>
 // (Held to 128 registers, so that more of a decode step's many short blocks share a CU, the compiler spills 400 to
 // 1,000 bytes a lane: what the tile's pipeline carries is more than that.  It is left its 233 to 256.)
 __global__ void __launch_bounds__(512)
@@ -524,7 +527,7 @@ gated_delta_kernel(const T* __restrict__ qkv, int qkv_stride, const T* __restric
                    int a_off, const float* __restrict__ A_log, const float* __restrict__ dt_bias,
                    float* __restrict__ state, long long state_stride, const int32_t* __restrict__ qo_indptr,
                    const int32_t* __restrict__ slot_ids, float* __restrict__ o_raw, int H, int G, int dk, int dv, int lpc,
-                   int col_groups) {
+                   int col_groups, const float* __restrict__ a_ch, int a_stride) {
   extern __shared__ __attribute__((aligned(16))) float lds[];
   // per token of the tile: k [dk], q [dk] (raw, then unit), v [kDeltaCols], o [kDeltaCols]; then six scalars
   const int dkp = dk + dk / 16 * 4;  // a token's keys in LDS: four floats of padding after every sixteen, so that
@@ -534,6 +537,7 @@ gated_delta_kernel(const T* __restrict__ qkv, int qkv_stride, const T* __restric
   float* v_l = q_l + kDeltaTile * dkp;
   float* o_l = v_l + kDeltaTile * kDeltaCols;
   float* sc_l = o_l + kDeltaTile * kDeltaCols;  // [kDeltaTile][6]: beta, decay, 1/|k|, scale/|q|, k^ . q^
+  float* g_l = sc_l + kDeltaTile * 6;           // (CH) [kDeltaTile][dkp]: a token's decays, padded as its key
   const int row = blockIdx.y;
   const int h = blockIdx.x / col_groups, cg = blockIdx.x % col_groups;
   const int g = h / (H / G);
@@ -556,7 +560,7 @@ gated_delta_kernel(const T* __restrict__ qkv, int qkv_stride, const T* __restric
 #pragma unroll
     for (int r = 0; r < kDeltaRows; ++r) S[r] = i0 + r < dk ? st[i0 + r] : 0.f;
   }
-  const float neg_rate = -expf(A_log[h]), bias = dt_bias[h];
+  const float neg_rate = -expf(A_log[h]), bias = CH ? 0.f : dt_bias[h];
   const float q_scale = 1.0f / sqrtf((float)dk);
   const int q_col = g * dk, k_col = G * dk + g * dk, v_col = 2 * G * dk + h * dv + cg * kDeltaCols;
   const int v_cols = min(kDeltaCols, dv - cg * kDeltaCols);
@@ -575,7 +579,7 @@ gated_delta_kernel(const T* __restrict__ qkv, int qkv_stride, const T* __restric
     if (threadIdx.x < nt) {
       const T* pr = proj + (size_t)(t0 + threadIdx.x) * proj_stride;
       pre_b = pr[b_off + h];
-      pre_a = pr[a_off + h];
+      if (!CH) pre_a = pr[a_off + h];
     }
     int tt = tt_first, d = d_first;
 #pragma unroll
@@ -615,7 +619,14 @@ gated_delta_kernel(const T* __restrict__ qkv, int qkv_stride, const T* __restric
     }
     if (threadIdx.x < nt) {
       sc_l[6 * threadIdx.x] = sigmoid_f(to_f32(pre_b));
-      sc_l[6 * threadIdx.x + 1] = expf(neg_rate * softplus_f(to_f32(pre_a) + bias));
+      if (!CH) sc_l[6 * threadIdx.x + 1] = expf(neg_rate * softplus_f(to_f32(pre_a) + bias));
+    }
+    if (CH) {
+      for (int e = threadIdx.x; e < nt * dk; e += n_threads) {
+        const int tt = e / dk, d = e % dk;
+        const float pre = a_ch[(size_t)(t0 + tt) * a_stride + h * dk + d] + dt_bias[h * dk + d];
+        g_l[tt * dkp + d + d / 16 * 4] = expf(neg_rate * softplus_f(pre));
+      }
     }
     if (t0 + kDeltaTile < end) fetch(t0 + kDeltaTile);  // on its way while this tile is worked on
     __syncthreads();
@@ -660,12 +671,17 @@ gated_delta_kernel(const T* __restrict__ qkv, int qkv_stride, const T* __restric
     // over the lane's rows and summed over the column's lanes together, and the state's update is no part of
     // the chain that o waits for.  A token's operands are read from LDS while the token before is worked on.
     struct Operands {
-      float kk[kDeltaRows], qq[kDeltaRows], v, beta, decay, kq;
+      float kk[kDeltaRows], qq[kDeltaRows], dd[CH ? kDeltaRows : 1], v, beta, decay, kq;
     };
     auto read = [&](Operands& x, int tt_raw) {
       const int tt = tt_raw < kDeltaTile ? tt_raw : kDeltaTile - 1;
       const float* kt = k_l + tt * dkp + i0 + i0 / 16 * 4;  // (i0 is a multiple of 16: a lane's rows have no padding between them)
       const float* qt = q_l + tt * dkp + i0 + i0 / 16 * 4;
+      if (CH) {
+        const float* gt = g_l + tt * dkp + i0 + i0 / 16 * 4;
+#pragma unroll
+        for (int r = 0; r < kDeltaRows; ++r) x.dd[r] = i0 + r < dk ? gt[r] : 0.f;
+      }
       if (VEC) {  // dk is a multiple of 4: four channels a read
 #pragma unroll
         for (int r = 0; r < kDeltaRows; r += 4) {
@@ -691,7 +707,7 @@ gated_delta_kernel(const T* __restrict__ qkv, int qkv_stride, const T* __restric
       float kv[4] = {0.f, 0.f, 0.f, 0.f}, sq[4] = {0.f, 0.f, 0.f, 0.f};
 #pragma unroll
       for (int r = 0; r < kDeltaRows; ++r) {
-        S[r] = x.decay * S[r];
+        S[r] = (CH ? x.dd[r] : x.decay) * S[r];
         kv[r % 4] = fmaf(S[r], x.kk[r], kv[r % 4]);
         sq[r % 4] = fmaf(S[r], x.qq[r], sq[r % 4]);
       }
@@ -739,13 +755,13 @@ gated_delta_kernel(const T* __restrict__ qkv, int qkv_stride, const T* __restric
 // ahead, few registers, so that many of these short blocks share a CU.  Every sum is taken in the order in which
 // gated_delta_kernel takes it (the norms by eight lanes over every eighth channel, the products with the state by
 // four chains a lane and then the column's lanes), so a token's result has the same bits from either kernel.
-template <typename T, bool VEC, int kDeltaRows>
+template <typename T, bool VEC, int kDeltaRows, bool CH>
 __global__ void __launch_bounds__(512)
 gated_delta_step_kernel(const T* __restrict__ qkv, int qkv_stride, const T* __restrict__ proj, int proj_stride, int b_off,
                         int a_off, const float* __restrict__ A_log, const float* __restrict__ dt_bias,
                         float* __restrict__ state, long long state_stride, const int32_t* __restrict__ qo_indptr,
                         const int32_t* __restrict__ slot_ids, float* __restrict__ o_raw, int H, int G, int dk, int dv,
-                        int lpc, int col_groups) {
+                        int lpc, int col_groups, const float* __restrict__ a_ch, int a_stride) {
   constexpr int kCols = 32;
   extern __shared__ __attribute__((aligned(16))) float lds[];
   const int dkp = dk + dk / 16 * 4;
@@ -778,8 +794,8 @@ gated_delta_step_kernel(const T* __restrict__ qkv, int qkv_stride, const T* __re
     for (int r = 0; r < kDeltaRows; ++r) S[r] = i0 + r < dk ? st[i0 + r] : 0.f;
   }
   const float v = to_f32(tok[2 * G * dk + h * dv + j]);
-  const float pb = to_f32(proj[t * proj_stride + b_off + h]), pa = to_f32(proj[t * proj_stride + a_off + h]);
-  const float neg_rate = -expf(A_log[h]), bias = dt_bias[h];
+  const float pb = to_f32(proj[t * proj_stride + b_off + h]), pa = CH ? 0.f : to_f32(proj[t * proj_stride + a_off + h]);
+  const float neg_rate = -expf(A_log[h]), bias = CH ? 0.f : dt_bias[h];
   __syncthreads();
   const int sub = threadIdx.x % 8;
   float kk2 = 0.f, qq2 = 0.f, kq = 0.f;
@@ -794,7 +810,7 @@ gated_delta_step_kernel(const T* __restrict__ qkv, int qkv_stride, const T* __re
   kq = row_group_sum(kq, 8);
   const float k_inv = 1.0f / sqrtf(kk2 + 1e-6f), q_inv = (1.0f / sqrtf((float)dk)) / sqrtf(qq2 + 1e-6f);
   const float kq_hat = kq * k_inv * q_inv;
-  const float beta = sigmoid_f(pb), decay = expf(neg_rate * softplus_f(pa + bias));
+  const float beta = sigmoid_f(pb), decay = CH ? 0.f : expf(neg_rate * softplus_f(pa + bias));
   float kv[4] = {0.f, 0.f, 0.f, 0.f}, sq[4] = {0.f, 0.f, 0.f, 0.f};
   float kk[kDeltaRows];
 #pragma unroll
@@ -803,7 +819,9 @@ gated_delta_step_kernel(const T* __restrict__ qkv, int qkv_stride, const T* __re
     const bool in = i < dk;
     kk[r] = in ? k_l[i + i / 16 * 4] * k_inv : 0.f;
     const float qq = in ? q_l[i + i / 16 * 4] * q_inv : 0.f;
-    S[r] = decay * S[r];
+    float dec = decay;
+    if (CH) dec = in ? expf(neg_rate * softplus_f(a_ch[t * a_stride + h * dk + i] + dt_bias[h * dk + i])) : 0.f;
+    S[r] = dec * S[r];
     kv[r % 4] = fmaf(S[r], kk[r], kv[r % 4]);
     sq[r % 4] = fmaf(S[r], qq, sq[r % 4]);
   }
@@ -826,23 +844,52 @@ gated_delta_step_kernel(const T* __restrict__ qkv, int qkv_stride, const T* __re
   }
 }
 
-// out[t, h, :] = T(o / sqrt(mean(o^2) + eps) * norm_w * silu(gate[t, h, :])): one wave a (token, head).
-template <typename T>
+// out[t, h, :] = T(o / sqrt(mean(o^2) + eps) * norm_w * act(gate[t, h, :])): one wave a (token, head).  act is silu
+// or (SIGMOID) the logistic function; the weight is one vector for all heads (w_stride 0) or a vector a head (dv).
+template <typename T, bool SIGMOID>
 __global__ void __launch_bounds__(kHeadWaves* kWave)
 delta_output_kernel(const float* __restrict__ o_raw, const T* __restrict__ proj, int proj_stride, int gate_off,
-                    const float* __restrict__ norm_w, float eps, T* __restrict__ out, int H, int dv) {
+                    const float* __restrict__ norm_w, int w_stride, float eps, T* __restrict__ out, int H, int dv,
+                    const float* __restrict__ den) {
   const int t = blockIdx.x;
   const int h = blockIdx.y * kHeadWaves + threadIdx.x / kWave;
   const int lane = threadIdx.x % kWave;
   if (h >= H) return;
   const float* o = o_raw + ((size_t)t * H + h) * dv;
+  // (den: every element of the head is first divided by the head's own number)
+  const float pre = den ? 1.0f / den[(size_t)t * H + h] : 1.0f;
   float ss = 0.f;
-  for (int d = lane; d < dv; d += kWave) ss = fmaf(o[d], o[d], ss);
+  for (int d = lane; d < dv; d += kWave) ss = fmaf(o[d] * pre, o[d] * pre, ss);
   ss = wave_sum(ss);
-  const float inv = 1.0f / sqrtf(ss / (float)dv + eps);
+  const float inv = pre / sqrtf(ss / (float)dv + eps);
   const T* gp = proj + (size_t)t * proj_stride + gate_off + (size_t)h * dv;
   T* op = out + ((size_t)t * H + h) * dv;
-  for (int d = lane; d < dv; d += kWave) op[d] = from_f32<T>(o[d] * inv * norm_w[d] * silu_f(to_f32(gp[d])));
+  const float* wp = norm_w + (size_t)h * w_stride;
+  for (int d = lane; d < dv; d += kWave) {
+    const float gate = to_f32(gp[d]);
+    op[d] = from_f32<T>(o[d] * inv * wp[d] * (SIGMOID ? sigmoid_f(gate) : silu_f(gate)));
+  }
+}
+
+// The same for rows of o_raw in units of 65535 tokens (a grid's first dimension).
+template <typename T>
+int launch_head_output(const float* o_raw, const T* gate, int gate_stride, int gate_off, const float* norm_w, int w_stride,
+                       float eps, T* out, int n_tokens, int H, int dv, bool sigmoid, hipStream_t stream,
+                       const float* den = nullptr) {
+  for (int t0 = 0; t0 < n_tokens; t0 += 65535) {
+    const int nt = n_tokens - t0 < 65535 ? n_tokens - t0 : 65535;
+    const dim3 ogrid(nt, (H + kHeadWaves - 1) / kHeadWaves);
+    const float* src = o_raw + (size_t)t0 * H * dv;
+    if (sigmoid)
+      delta_output_kernel<T, true><<<ogrid, kHeadWaves * kWave, 0, stream>>>(src, gate + (size_t)t0 * gate_stride, gate_stride, gate_off,
+                                                                             norm_w, w_stride, eps, out + (size_t)t0 * H * dv, H, dv,
+                                                                             den ? den + (size_t)t0 * H : nullptr);
+    else
+      delta_output_kernel<T, false><<<ogrid, kHeadWaves * kWave, 0, stream>>>(src, gate + (size_t)t0 * gate_stride, gate_stride, gate_off,
+                                                                              norm_w, w_stride, eps, out + (size_t)t0 * H * dv, H, dv,
+                                                                             den ? den + (size_t)t0 * H : nullptr);
+  }
+  return tl_check_launch("head_output");
 }
 
 }  // namespace
@@ -1034,16 +1081,21 @@ TL_EXPORT int tl_selective_scan(const void* x, const void* dt_pre, int dt_dtype,
 }
 
 // qkv, proj, out as the kernels describe; state: S^T of head h at state + slot * state_stride + h * dv * dk;
-// o_raw: workspace of n_tokens * H * dv floats.
+// o_raw: workspace of n_tokens * H * dv floats.  gate: the matrix whose H * dv columns from gate_off hold the output
+// gate (proj itself, or a tensor of its own); gate_sigmoid: the gate's activation is the logistic function, not silu.
+// a_ch (or null): 32-bit pre-activations of a decay per key channel, [n_tokens, a_stride] with H * dk columns; then
+// dt_bias has H * dk entries.
 TL_EXPORT int tl_gated_delta(const void* qkv, int qkv_stride, const void* proj, int proj_stride, int gate_off, int b_off,
                              int a_off, const float* A_log, const float* dt_bias, const float* norm_w, float eps, float* state,
                              long long state_stride, const int32_t* qo_indptr, const int32_t* slot_ids, void* out, int n_tokens,
-                             int n_seqs, int H, int G, int dk, int dv, float* o_raw, int dtype, hipStream_t stream) {
+                             int n_seqs, int H, int G, int dk, int dv, float* o_raw, int dtype, const void* gate, int gate_stride,
+                             int gate_sigmoid, const float* a_ch, int a_stride, hipStream_t stream) {
   TL_REQUIRE(n_seqs >= 0 && n_tokens >= 0 && H > 0 && G > 0 && dk > 0 && dv > 0, "gated_delta: bad sizes");
   TL_REQUIRE(H % G == 0, "gated_delta: %d heads are not a multiple of %d key heads", H, G);
   if (dk > 256) return tl_fail(TL_ERR_UNSUPPORTED, "gated_delta: keys of %d channels, at most 256", dk);
   TL_REQUIRE(n_seqs <= 65535 && n_tokens <= 0x7fffffff / 4, "gated_delta: too many requests or tokens a step");
-  TL_REQUIRE(o_raw != nullptr, "gated_delta: no workspace");
+  TL_REQUIRE(o_raw != nullptr && gate != nullptr, "gated_delta: no workspace or no gate");
+  TL_REQUIRE(a_ch == nullptr || a_stride >= H * dk, "gated_delta: rows of %d decays, %d needed", a_stride, H * dk);
   if (n_seqs == 0 || n_tokens == 0) return TL_OK;
   if (dtype != TL_F32 && dtype != TL_BF16) return tl_fail(TL_ERR_ARG, "gated_delta: unknown dtype %d", dtype);
   const int rows = dk <= 128 ? 8 : 16;
@@ -1051,66 +1103,321 @@ TL_EXPORT int tl_gated_delta(const void* qkv, int qkv_stride, const void* proj, 
   while (rows * lpc < dk) lpc *= 2;  // at most 16: a column's lanes lie in one row of 16 lanes
   // columns a block: 16 while that leaves fewer than two blocks a CU, else 32 (a step of single tokens: always 32)
   const bool single = n_tokens == n_seqs;
+  const bool ch = a_ch != nullptr;
   const int cols = !single && (long long)n_seqs * H * ((dv + 15) / 16) < 2LL * tl_device_facts().compute_units ? 16 : 32;
   const int threads = (cols * lpc + kWave - 1) / kWave * kWave;
   const int col_groups = (dv + cols - 1) / cols;
-  const size_t lds = ((size_t)kDeltaTile * (2 * (dk + dk / 16 * 4) + 2 * cols + 6)) * sizeof(float);
+  const int dkp = dk + dk / 16 * 4;
+  const size_t lds = ((size_t)kDeltaTile * (2 * dkp + 2 * cols + 6 + (ch ? dkp : 0))) * sizeof(float);
   const dim3 grid(H * col_groups, n_seqs);
-#define TL_DELTA_R(T, VEC, R, C)                                                                                       \
-  gated_delta_kernel<T, VEC, R, C><<<grid, threads, lds, stream>>>((const T*)qkv, qkv_stride, (const T*)proj, proj_stride, b_off, \
-                                                                   a_off, A_log, dt_bias, state, state_stride, qo_indptr, slot_ids, \
-                                                                   o_raw, H, G, dk, dv, lpc, col_groups)
-#define TL_DELTA(T, VEC)                                \
-  do {                                                  \
-    if (rows == 8 && cols == 16) TL_DELTA_R(T, VEC, 8, 16);   \
-    else if (rows == 8) TL_DELTA_R(T, VEC, 8, 32);      \
-    else if (cols == 16) TL_DELTA_R(T, VEC, 16, 16);    \
-    else TL_DELTA_R(T, VEC, 16, 32);                    \
+#define TL_DELTA_R(T, VEC, R, C, CH)                                                                                   \
+  gated_delta_kernel<T, VEC, R, C, CH><<<grid, threads, lds, stream>>>(                                                \
+      (const T*)qkv, qkv_stride, (const T*)proj, proj_stride, b_off, a_off, A_log, dt_bias, state, state_stride,       \
+      qo_indptr, slot_ids, o_raw, H, G, dk, dv, lpc, col_groups, a_ch, a_stride)
+#define TL_DELTA(T, VEC, CH)                                      \
+  do {                                                            \
+    if (rows == 8 && cols == 16) TL_DELTA_R(T, VEC, 8, 16, CH);   \
+    else if (rows == 8) TL_DELTA_R(T, VEC, 8, 32, CH);            \
+    else if (cols == 16) TL_DELTA_R(T, VEC, 16, 16, CH);          \
+    else TL_DELTA_R(T, VEC, 16, 32, CH);                          \
   } while (0)
   // four rows a load where every lane's rows start at a multiple of 16 bytes, in LDS and in the state
   const bool vec = dk % 4 == 0 && ((uintptr_t)state % 16) == 0 && state_stride % 4 == 0;
-#define TL_DELTA_STEP(T, VEC)                                                                                          \
+#define TL_DELTA_STEP(T, VEC, CH)                                                                                      \
   do {                                                                                                                 \
-    const size_t step_lds = 2 * (size_t)(dk + dk / 16 * 4) * sizeof(float);                                            \
+    const size_t step_lds = 2 * (size_t)dkp * sizeof(float);                                                           \
     if (rows == 8)                                                                                                     \
-      gated_delta_step_kernel<T, VEC, 8><<<grid, threads, step_lds, stream>>>(                                         \
+      gated_delta_step_kernel<T, VEC, 8, CH><<<grid, threads, step_lds, stream>>>(                                     \
           (const T*)qkv, qkv_stride, (const T*)proj, proj_stride, b_off, a_off, A_log, dt_bias, state, state_stride,   \
-          qo_indptr, slot_ids, o_raw, H, G, dk, dv, lpc, col_groups);                                                  \
+          qo_indptr, slot_ids, o_raw, H, G, dk, dv, lpc, col_groups, a_ch, a_stride);                                  \
     else                                                                                                               \
-      gated_delta_step_kernel<T, VEC, 16><<<grid, threads, step_lds, stream>>>(                                        \
+      gated_delta_step_kernel<T, VEC, 16, CH><<<grid, threads, step_lds, stream>>>(                                    \
           (const T*)qkv, qkv_stride, (const T*)proj, proj_stride, b_off, a_off, A_log, dt_bias, state, state_stride,   \
-          qo_indptr, slot_ids, o_raw, H, G, dk, dv, lpc, col_groups);                                                  \
+          qo_indptr, slot_ids, o_raw, H, G, dk, dv, lpc, col_groups, a_ch, a_stride);                                  \
   } while (0)
-  if (single) {
-    if (dtype == TL_F32) {
-      if (vec) TL_DELTA_STEP(float, true);
-      else TL_DELTA_STEP(float, false);
-    } else {
-      if (vec) TL_DELTA_STEP(bf16_t, true);
-      else TL_DELTA_STEP(bf16_t, false);
-    }
-  } else if (dtype == TL_F32) {
-    if (vec) TL_DELTA(float, true);
-    else TL_DELTA(float, false);
-  } else {
-    if (vec) TL_DELTA(bf16_t, true);
-    else TL_DELTA(bf16_t, false);
-  }
+#define TL_DELTA_ANY(T, VEC, CH)          \
+  do {                                    \
+    if (single) TL_DELTA_STEP(T, VEC, CH); \
+    else TL_DELTA(T, VEC, CH);            \
+  } while (0)
+#define TL_DELTA_T(T)                            \
+  do {                                           \
+    if (vec && ch) TL_DELTA_ANY(T, true, true);  \
+    else if (vec) TL_DELTA_ANY(T, true, false);  \
+    else if (ch) TL_DELTA_ANY(T, false, true);   \
+    else TL_DELTA_ANY(T, false, false);          \
+  } while (0)
+  if (dtype == TL_F32) TL_DELTA_T(float);
+  else TL_DELTA_T(bf16_t);
+#undef TL_DELTA_T
+#undef TL_DELTA_ANY
 #undef TL_DELTA_STEP
 #undef TL_DELTA
 #undef TL_DELTA_R
   int rc = tl_check_launch("gated_delta");
   if (rc != TL_OK) return rc;
-  for (int t0 = 0; t0 < n_tokens; t0 += 65535) {
-    const int nt = n_tokens - t0 < 65535 ? n_tokens - t0 : 65535;
-    const dim3 ogrid(nt, (H + kHeadWaves - 1) / kHeadWaves);
-    const float* src = o_raw + (size_t)t0 * H * dv;
-    if (dtype == TL_F32)
-      delta_output_kernel<float><<<ogrid, kHeadWaves * kWave, 0, stream>>>(
-          src, (const float*)proj + (size_t)t0 * proj_stride, proj_stride, gate_off, norm_w, eps, (float*)out + (size_t)t0 * H * dv, H, dv);
-    else
-      delta_output_kernel<bf16_t><<<ogrid, kHeadWaves * kWave, 0, stream>>>(
-          src, (const bf16_t*)proj + (size_t)t0 * proj_stride, proj_stride, gate_off, norm_w, eps, (bf16_t*)out + (size_t)t0 * H * dv, H, dv);
+  if (dtype == TL_F32)
+    return launch_head_output<float>(o_raw, (const float*)gate, gate_stride, gate_off, norm_w, 0, eps, (float*)out, n_tokens, H, dv,
+                                     gate_sigmoid != 0, stream);
+  return launch_head_output<bf16_t>(o_raw, (const bf16_t*)gate, gate_stride, gate_off, norm_w, 0, eps, (bf16_t*)out, n_tokens, H, dv,
+                                    gate_sigmoid != 0, stream);
+}
+
+
+// ============================================================================= matrix memory (mLSTM)
+// Per request and head h, in 32-bit: a matrix C [dk][dv], a vector n [dk] and a running maximum m (all zero at the
+// start).  For every token, with q already times dk^-1/2, the log input gate i = cap tanh((i~ + b_i) / cap) and the
+// log forget gate f = logsigmoid(cap tanh((f~ + b_f) / cap)):
+//   m' = max(f + m, i);  keep = exp(f + m - m');  take = exp(i - m')
+//   C <- keep C + take k v^T;  n <- keep n + take k;  o = C^T q / (max(|n . q|, exp(-m')) + 1e-6)
+// n is the matrix's column dv (its "value" is 1), so the state of a head is [dv + 1][dk], column by column, and
+// behind all heads' columns lies m, once for every column (the blocks that share a head each keep their own).
+// A block takes kMemCols columns of one (request, head); lpc neighbouring lanes share a column, each holding R rows.
+// The tokens come in tiles of kDeltaTile: the next tile's raw q, k, v and gates travel into registers while this one
+// is worked on; one wave walks the tile's maxima (a chain of additions and comparisons, no exponentials on it)
+// and then takes the exponentials side by side; the keys go to LDS times `take`, so a token costs a lane three
+// operations a row.  The numerators go to o_raw [n, H, dv], the denominators to den [n, H].
+namespace {
+constexpr int kMemCols = 32;
+
+__device__ __forceinline__ float log_sigmoid_f(float z) { return fminf(z, 0.f) - log1pf(expf(-fabsf(z))); }
+
+template <typename T, bool VEC, int R>
+__global__ void __launch_bounds__(512)
+matrix_memory_kernel(const T* __restrict__ proj, int stride, int q_off, int k_off, int v_off, int i_off, int f_off,
+                     const float* __restrict__ i_bias, const float* __restrict__ f_bias, float cap,
+                     float* __restrict__ state, long long state_stride, const int32_t* __restrict__ qo_indptr,
+                     const int32_t* __restrict__ slot_ids, float* __restrict__ o_raw, float* __restrict__ den, int H, int dk,
+                     int dv, int lpc, int col_groups) {
+  extern __shared__ __attribute__((aligned(16))) float lds[];
+  const int dkp = dk + dk / 16 * 4;
+  float* k_l = lds;
+  float* q_l = k_l + kDeltaTile * dkp;
+  float* v_l = q_l + kDeltaTile * dkp;
+  float* o_l = v_l + kDeltaTile * kMemCols;
+  float* sc_l = o_l + kDeltaTile * kMemCols;  // [kDeltaTile][4]: keep, take, exp(-m'); then the maximum that enters the next tile
+  const int W = dv + 1;
+  const int row = blockIdx.y;
+  const int h = blockIdx.x / col_groups, cg = blockIdx.x % col_groups;
+  const int start = qo_indptr[row], end = qo_indptr[row + 1];
+  const int n_threads = blockDim.x;
+  const int j_loc = threadIdx.x / lpc, part = threadIdx.x % lpc;
+  const int j_raw = cg * kMemCols + j_loc;
+  const bool live = j_loc < kMemCols && j_raw < W;
+  const int j = j_raw < W ? j_raw : W - 1;
+  const bool norm_col = j == dv;
+  const int i0 = part * R;
+  float* slot = state + (long long)slot_ids[row] * state_stride;
+  float* st = slot + ((size_t)h * W + j) * dk;
+  float* m_at = slot + (size_t)H * W * dk + (size_t)h * W + j;
+  float S[R];
+  if (VEC) {
+#pragma unroll
+    for (int r = 0; r < R; r += 4) {
+      const float4 s4 = i0 + r < dk ? *reinterpret_cast<const float4*>(st + i0 + r) : float4{0.f, 0.f, 0.f, 0.f};
+      S[r] = s4.x; S[r + 1] = s4.y; S[r + 2] = s4.z; S[r + 3] = s4.w;
+    }
+  } else {
+#pragma unroll
+    for (int r = 0; r < R; ++r) S[r] = i0 + r < dk ? st[i0 + r] : 0.f;
   }
-  return tl_check_launch("delta_output");
+  if (threadIdx.x == 0) sc_l[4 * kDeltaTile] = *m_at;  // (thread 0 holds a live column: cg * kMemCols < W)
+  const float q_scale = 1.0f / sqrtf((float)dk);
+  const float bi = i_bias[h], bf = f_bias[h];
+  const int v_cols = min(kMemCols, W - cg * kMemCols);  // (the normaliser's column included)
+  const int v_col = v_off + h * dv + cg * kMemCols;
+
+  const int two_dk = 2 * dk;
+  const int tt_first = threadIdx.x / two_dk, d_first = threadIdx.x % two_dk;
+  const int tt_step = n_threads / two_dk, d_step = n_threads % two_dk;
+  constexpr int kPreKQ = R, kPreV = 8;
+  T pre_kq[kPreKQ], pre_v[kPreV], pre_i = from_f32<T>(0.f), pre_f = from_f32<T>(0.f);
+  auto fetch = [&](int t0) {
+    const int nt = min(kDeltaTile, end - t0);
+    if (threadIdx.x < nt) {
+      const T* pr = proj + (size_t)(t0 + threadIdx.x) * stride;
+      pre_i = pr[i_off + h];
+      pre_f = pr[f_off + h];
+    }
+    int tt = tt_first, d = d_first;
+#pragma unroll
+    for (int u = 0; u < kPreKQ; ++u) {
+      if (tt < nt) pre_kq[u] = proj[(size_t)(t0 + tt) * stride + (d < dk ? k_off + h * dk + d : q_off + h * dk + d - dk)];
+      tt += tt_step;
+      d += d_step;
+      if (d >= two_dk) { d -= two_dk; ++tt; }
+    }
+#pragma unroll
+    for (int u = 0; u < kPreV; ++u) {
+      const int e = threadIdx.x + u * n_threads;
+      const int tt = e / kMemCols, d = e % kMemCols;
+      if (tt < nt && d < v_cols && cg * kMemCols + d < dv) pre_v[u] = proj[(size_t)(t0 + tt) * stride + v_col + d];
+    }
+  };
+  if (start < end) fetch(start);
+  for (int t0 = start; t0 < end; t0 += kDeltaTile) {
+    const int nt = min(kDeltaTile, end - t0);
+    __syncthreads();  // the tile before has been read to its end
+    if (threadIdx.x < kWave) {
+      // the gates of the tile's tokens, a lane a token; then the maxima, every lane walking the same chain
+      const int lane = threadIdx.x;
+      float gi = 0.f, gf = 0.f;
+      if (lane < nt) {
+        gi = cap * tanhf((to_f32(pre_i) + bi) / cap);
+        gf = log_sigmoid_f(cap * tanhf((to_f32(pre_f) + bf) / cap));
+      }
+      float m = sc_l[4 * kDeltaTile], m_before = 0.f, m_mine = 0.f;
+      for (int tt = 0; tt < nt; ++tt) {
+        const float ft = __shfl(gf, tt, kWave), it = __shfl(gi, tt, kWave);
+        const float m_new = fmaxf(ft + m, it);
+        if (lane == tt) { m_before = m; m_mine = m_new; }
+        m = m_new;
+      }
+      if (lane < nt) {
+        sc_l[4 * lane] = expf(gf + m_before - m_mine);
+        sc_l[4 * lane + 1] = expf(gi - m_mine);
+        sc_l[4 * lane + 2] = expf(-m_mine);
+      }
+      if (lane == 0) sc_l[4 * kDeltaTile] = m;
+    }
+    __syncthreads();
+    {
+      int tt = tt_first, d = d_first;
+#pragma unroll
+      for (int u = 0; u < kPreKQ; ++u) {
+        const int dd = d < dk ? d : d - dk;
+        if (tt < nt) (d < dk ? k_l : q_l)[tt * dkp + dd + dd / 16 * 4] = to_f32(pre_kq[u]) * (d < dk ? sc_l[4 * tt + 1] : q_scale);
+        tt += tt_step;
+        d += d_step;
+        if (d >= two_dk) { d -= two_dk; ++tt; }
+      }
+    }
+#pragma unroll
+    for (int u = 0; u < kPreV; ++u) {
+      const int e = threadIdx.x + u * n_threads;
+      const int tt = e / kMemCols, d = e % kMemCols;
+      if (tt < nt && d < v_cols) v_l[tt * kMemCols + d] = cg * kMemCols + d < dv ? to_f32(pre_v[u]) : 1.0f;
+    }
+    if (t0 + kDeltaTile < end) fetch(t0 + kDeltaTile);  // on its way while this tile is worked on
+    __syncthreads();
+    struct Operands {
+      float kk[R], qq[R], v, keep, floor;
+    };
+    auto read = [&](Operands& x, int tt_raw) {
+      const int tt = tt_raw < kDeltaTile ? tt_raw : kDeltaTile - 1;
+      const float* kt = k_l + tt * dkp + i0 + i0 / 16 * 4;
+      const float* qt = q_l + tt * dkp + i0 + i0 / 16 * 4;
+      if (VEC) {
+#pragma unroll
+        for (int r = 0; r < R; r += 4) {
+          const bool in = i0 + r < dk;
+          const float4 k4 = in ? *reinterpret_cast<const float4*>(kt + r) : float4{0.f, 0.f, 0.f, 0.f};
+          const float4 q4 = in ? *reinterpret_cast<const float4*>(qt + r) : float4{0.f, 0.f, 0.f, 0.f};
+          x.kk[r] = k4.x; x.kk[r + 1] = k4.y; x.kk[r + 2] = k4.z; x.kk[r + 3] = k4.w;
+          x.qq[r] = q4.x; x.qq[r + 1] = q4.y; x.qq[r + 2] = q4.z; x.qq[r + 3] = q4.w;
+        }
+      } else {
+#pragma unroll
+        for (int r = 0; r < R; ++r) {
+          x.kk[r] = i0 + r < dk ? kt[r] : 0.f;
+          x.qq[r] = i0 + r < dk ? qt[r] : 0.f;
+        }
+      }
+      x.v = v_l[tt * kMemCols + (j_loc < kMemCols ? j_loc : 0)];
+      x.keep = sc_l[4 * tt];
+      x.floor = sc_l[4 * tt + 2];
+    };
+    auto token = [&](const Operands& x, int tt) {
+      float sq[4] = {0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+      for (int r = 0; r < R; ++r) {
+        S[r] = fmaf(x.kk[r], x.v, x.keep * S[r]);
+        sq[r % 4] = fmaf(S[r], x.qq[r], sq[r % 4]);
+      }
+      const float sq_all = row_group_sum((sq[0] + sq[1]) + (sq[2] + sq[3]), lpc);
+      if (live && part == 0) o_l[tt * kMemCols + j_loc] = norm_col ? fmaxf(fabsf(sq_all), x.floor) + 1e-6f : sq_all;
+    };
+    Operands xa, xb;
+    read(xa, 0);
+#pragma unroll 1
+    for (int tt = 0; tt < nt; tt += 2) {
+      read(xb, tt + 1);
+      token(xa, tt);
+      if (tt + 1 < nt) {
+        read(xa, tt + 2);
+        token(xb, tt + 1);
+      }
+    }
+    __syncthreads();
+    for (int e = threadIdx.x; e < nt * kMemCols; e += n_threads) {
+      const int tt = e / kMemCols, d = e % kMemCols;
+      if (d < v_cols) {
+        const int col = cg * kMemCols + d;
+        if (col < dv) o_raw[((size_t)(t0 + tt) * H + h) * dv + col] = o_l[e];
+        else den[(size_t)(t0 + tt) * H + h] = o_l[e];
+      }
+    }
+  }
+  __syncthreads();
+  if (live) {
+    if (VEC) {
+#pragma unroll
+      for (int r = 0; r < R; r += 4)
+        if (i0 + r < dk) *reinterpret_cast<float4*>(st + i0 + r) = float4{S[r], S[r + 1], S[r + 2], S[r + 3]};
+    } else {
+#pragma unroll
+      for (int r = 0; r < R; ++r)
+        if (i0 + r < dk) st[i0 + r] = S[r];
+    }
+    if (part == 0) *m_at = sc_l[4 * kDeltaTile];
+  }
+}
+}  // namespace
+
+// proj [n_tokens, stride]: the columns of q (H * dk from q_off), k, v (H * dv) and of the two gates' pre-activations
+// (H each) of one matrix.  state: per slot H * (dv + 1) * dk + H * (dv + 1) floats.  gate [n_tokens, gate_stride]:
+// the output gate's H * dv columns from gate_off.  norm_w: H * dv floats.  o_raw, den: workspaces of n_tokens * H * dv
+// and n_tokens * H floats.  out [n_tokens, H * dv] = T(o / rms(o) * norm_w * sigmoid(gate)).
+TL_EXPORT int tl_matrix_memory(const void* proj, int stride, int q_off, int k_off, int v_off, int i_off, int f_off,
+                               const float* i_bias, const float* f_bias, float cap, const void* gate, int gate_stride,
+                               int gate_off, const float* norm_w, float eps, float* state, long long state_stride,
+                               const int32_t* qo_indptr, const int32_t* slot_ids, void* out, int n_tokens, int n_seqs, int H,
+                               int dk, int dv, float* o_raw, float* den, int dtype, hipStream_t stream) {
+  TL_REQUIRE(n_seqs >= 0 && n_tokens >= 0 && H > 0 && dk > 0 && dv > 0 && cap > 0.f, "matrix_memory: bad sizes");
+  if (dk > 256) return tl_fail(TL_ERR_UNSUPPORTED, "matrix_memory: keys of %d channels, at most 256", dk);
+  TL_REQUIRE(n_seqs <= 65535 && n_tokens <= 0x7fffffff / 4, "matrix_memory: too many requests or tokens a step");
+  TL_REQUIRE(o_raw != nullptr && den != nullptr && gate != nullptr, "matrix_memory: no workspace or no gate");
+  if (n_seqs == 0 || n_tokens == 0) return TL_OK;
+  if (dtype != TL_F32 && dtype != TL_BF16) return tl_fail(TL_ERR_ARG, "matrix_memory: unknown dtype %d", dtype);
+  const int rows = dk <= 128 ? 8 : 16;
+  int lpc = 1;
+  while (rows * lpc < dk) lpc *= 2;
+  const int threads = (kMemCols * lpc + kWave - 1) / kWave * kWave;
+  const int col_groups = (dv + 1 + kMemCols - 1) / kMemCols;
+  const int dkp = dk + dk / 16 * 4;
+  const size_t lds = ((size_t)kDeltaTile * (2 * dkp + 2 * kMemCols + 4) + 4) * sizeof(float);
+  const dim3 grid(H * col_groups, n_seqs);
+  const bool vec = dk % 4 == 0 && ((uintptr_t)state % 16) == 0 && state_stride % 4 == 0;
+#define TL_MEM(T, VEC, R)                                                                                               \
+  matrix_memory_kernel<T, VEC, R><<<grid, threads, lds, stream>>>((const T*)proj, stride, q_off, k_off, v_off, i_off, f_off, \
+                                                                  i_bias, f_bias, cap, state, state_stride, qo_indptr,  \
+                                                                  slot_ids, o_raw, den, H, dk, dv, lpc, col_groups)
+#define TL_MEM_T(T)                                  \
+  do {                                               \
+    if (vec && rows == 8) TL_MEM(T, true, 8);        \
+    else if (vec) TL_MEM(T, true, 16);               \
+    else if (rows == 8) TL_MEM(T, false, 8);         \
+    else TL_MEM(T, false, 16);                       \
+  } while (0)
+  if (dtype == TL_F32) TL_MEM_T(float);
+  else TL_MEM_T(bf16_t);
+#undef TL_MEM_T
+#undef TL_MEM
+  int rc = tl_check_launch("matrix_memory");
+  if (rc != TL_OK) return rc;
+  if (dtype == TL_F32)
+    return launch_head_output<float>(o_raw, (const float*)gate, gate_stride, gate_off, norm_w, dv, eps, (float*)out, n_tokens, H, dv,
+                                     true, stream, den);
+  return launch_head_output<bf16_t>(o_raw, (const bf16_t*)gate, gate_stride, gate_off, norm_w, dv, eps, (bf16_t*)out, n_tokens, H, dv,
+                                    true, stream, den);
 }

@@ -37,6 +37,7 @@ CORE_SOURCES = [
     "sampling.hip",
     "sequence_ops.hip",
     "head_ops.hip",
+    "routed_ops.hip",
 ]
 HEADERS = ["common.h", "qkv_epilogue.h", "no_alloc.h"]
 

@@ -40,7 +40,14 @@ _CORE_SIGNATURES = {
     "tl_rope_norm_kv_write": [_P, _I, _I, _I, _I, _I, _P, _I, _I, _F, _P, _P, _P, _I, _I, _P],
     "tl_causal_conv": [_P, _I, _P, _P, _P, _I64, _P, _P, _P, _P, _I, _I, _I, _I, _I, _I, _I, _P],
     "tl_selective_scan": [_P, _P, _I, _P, _I, _I, _I, _P, _I, _P, _P, _P, _P, _I64, _P, _P, _P, _I, _I, _I, _I, _P, _P, _I, _P, _P, _P],
-    "tl_gated_delta": [_P, _I, _P, _I, _I, _I, _I, _P, _P, _P, _F, _P, _I64, _P, _P, _P, _I, _I, _I, _I, _I, _I, _P, _I, _P],
+    "tl_gated_delta": [_P, _I, _P, _I, _I, _I, _I, _P, _P, _P, _F, _P, _I64, _P, _P, _P, _I, _I, _I, _I, _I, _I, _P, _I, _P, _I, _I, _P, _I, _P],
+    "tl_matrix_memory": [_P, _I, _I, _I, _I, _I, _I, _P, _P, _F, _P, _I, _I, _P, _F, _P, _I64, _P, _P, _P, _I, _I, _I, _I, _I, _P, _P, _I, _P],
+    "tl_router_topk": [_P, _I, _P, _I, _I, _I, _P, _P, _P],
+    "tl_expert_glu_pairs": [_P, _P, _P, _I, _I, _P, _I, _I, _I, _I, _P],
+    "tl_expert_down_pairs": [_P, _P, _P, _P, _I, _I, _P, _P, _P, _I, _P, _I, _I, _I, _I, _P],
+    "tl_bias_gelu": [_P, _P, _I, _I, _I, _P],
+    "tl_weighted_pair": [_P, _F, _P, _F, _P, _I64, _I, _P],
+    "tl_post_norm_add_norm": [_P, _P, _P, _F, _P, _F, _P, _I, _I, _I, _P],
     "tl_head_prepare": [_P, _I, _I, _I, _I, _I, _I, _P, _P, _P, _I, _F, _P, _I, _I, _I, _P, _F, _I, _P, _I, _P, _P, _P, _P, _I, _I, _P],
     "tl_branch_norm_add": [_P, _P, _P, _P, _I, _I, _F, _I, _P],
     "tl_rmsnorm_columns": [_P, _I, _I, _P, _P, _P, _I, _I, _I, _I, _F, _P],

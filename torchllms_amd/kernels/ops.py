@@ -10,9 +10,11 @@ a module's own helpers and tables stay in the module.
 ``products``         matrix products and the measurement that picks their kernel
 ``attention_ops``    plain, decode and prefill attention with their launch plans
 ``sequence_ops``     layer norm with a scaled sum, gated activations, unit-norm rotation with the cache
-                     write, short convolutions, selective scan, gated delta rule
+                     write, short convolutions, selective scan, gated delta rule, matrix memory
 ``head_ops``         branches normed into a 32-bit stream, heads prepared before the scores (weighted norm, partial
                      rotation, query factor, mixed values), gates, packing for attention through a latent, logit cap
+``routed_ops``       router (softmax scores, corrected choice), experts a (token, choice) at a time, bias with the
+                     exact gelu, the norm behind a branch together with the norm before the next
 ``sampling_ops``     the sampling kernel
 """
 
@@ -100,6 +102,8 @@ from .sequence_ops import (  # noqa: F401
     gated_delta,
     gelu_mul,
     layernorm,
+    matrix_memory,
+    matrix_memory_state_size,
     rope_norm_kv_write,
     selective_scan,
     state_region,
@@ -113,6 +117,15 @@ from .head_ops import (  # noqa: F401
     sigmoid_gate_,
     softcap_,
     unpack_heads_gate,
+)
+from .routed_ops import (  # noqa: F401
+    ROUTER_MAX_OUTPUTS,
+    bias_gelu_,
+    expert_down_pairs,
+    expert_glu_pairs,
+    post_norm_add_norm,
+    router_topk,
+    weighted_pair,
 )
 from .sampling_ops import (  # noqa: F401
     philox_uniform,

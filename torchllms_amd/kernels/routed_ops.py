@@ -1,0 +1,146 @@
+"""Kernels of a routed feed-forward (router with softmax scores and a correction for the choice, experts a
+(token, choice) at a time, experts that hand their input through, a shared expert with a gate), of a dense
+feed-forward with biases and the exact gelu, and of layers with a norm on either side of every branch."""
+
+from __future__ import annotations
+
+from typing import Optional, Tuple
+
+import torch
+
+from .base import KernelError, _gpu, _ptr, _stream, check, core, dtype_code
+
+#: the most outputs a router may have (experts and experts that hand their input through together)
+ROUTER_MAX_OUTPUTS = 512
+
+
+def router_topk(z: torch.Tensor, n_out: int, correction: torch.Tensor, top: int) -> Tuple[torch.Tensor, torch.Tensor]:
+    """``z`` float32 [n, >= n_out]: the router's outputs in the first ``n_out`` columns.  ``s = softmax(z)``; the
+    ``top`` outputs with the largest ``s + correction`` are chosen (of equal ones the lower index).  Returns
+    ``(ids int32 [n, top], weights float32 [n, top])``, the weights being the chosen outputs' ``s``."""
+    _gpu(z, correction)
+    if z.dim() != 2 or z.dtype != torch.float32 or z.stride(1) != 1 or z.shape[1] < n_out:
+        raise KernelError(f"router_topk: z must be float32 [n, >= {n_out}] with contiguous rows")
+    if tuple(correction.shape) != (n_out,) or correction.dtype != torch.float32 or not correction.is_contiguous():
+        raise KernelError(f"router_topk: correction must be a float32 vector of {n_out} entries")
+    if not 0 < top <= n_out:
+        raise KernelError(f"router_topk: {top} choices among {n_out} outputs")
+    n = z.shape[0]
+    ids = torch.empty((n, top), dtype=torch.int32, device=z.device)
+    weights = torch.empty((n, top), dtype=torch.float32, device=z.device)
+    check(core().tl_router_topk(z.data_ptr(), z.stride(0), correction.data_ptr(), n, n_out, top, ids.data_ptr(), weights.data_ptr(),
+                                _stream()))
+    return ids, weights
+
+
+def _pairs(x, ids, n_experts):
+    if x.dim() != 2 or not x.is_contiguous():
+        raise KernelError("routed experts: x must be a contiguous [n, D] matrix")
+    if ids.dim() != 2 or ids.shape[0] != x.shape[0] or ids.dtype != torch.int32 or not ids.is_contiguous():
+        raise KernelError("routed experts: ids must be contiguous int32 [n, top]")
+    if n_experts < 0:
+        raise KernelError("routed experts: a negative number of experts")
+
+
+def expert_glu_pairs(x: torch.Tensor, w_gate_up: torch.Tensor, ids: torch.Tensor) -> torch.Tensor:
+    """``mid[t, j] = silu(Wg[e] x[t]) * (Wu[e] x[t])`` with ``e = ids[t, j]``, for every pair whose ``e`` is below
+    the number of experts ``w_gate_up`` [E, 2F, D] holds (gate rows, then up rows); the others are left unwritten.
+    Returns [n, top, F] of x's dtype."""
+    _gpu(x, w_gate_up, ids)
+    E = w_gate_up.shape[0] if w_gate_up.dim() == 3 else -1
+    _pairs(x, ids, E)
+    n, D = x.shape
+    if w_gate_up.dim() != 3 or w_gate_up.shape[2] != D or w_gate_up.shape[1] % 2 or w_gate_up.dtype != x.dtype or not w_gate_up.is_contiguous():
+        raise KernelError(f"expert_glu_pairs: weights must be contiguous [E, 2F, {D}] of x's dtype")
+    F = w_gate_up.shape[1] // 2
+    top = ids.shape[1]
+    mid = torch.empty((n, top, F), dtype=x.dtype, device=x.device)
+    check(core().tl_expert_glu_pairs(x.data_ptr(), w_gate_up.data_ptr(), ids.data_ptr(), top, E, mid.data_ptr(), n, D, F,
+                                     dtype_code(x.dtype), _stream()))
+    return mid
+
+
+def expert_down_pairs(
+    mid: torch.Tensor,
+    w_down: torch.Tensor,
+    ids: torch.Tensor,
+    weights: torch.Tensor,
+    x: torch.Tensor,
+    shared: Optional[torch.Tensor] = None,
+    shared_gate: Optional[torch.Tensor] = None,
+) -> torch.Tensor:
+    """``out[t] = sum_j weights[t, j] * (Wd[e] mid[t, j] if e = ids[t, j] is an expert of w_down [E, D, F], else x[t])``,
+    plus ``sigmoid(shared_gate[t]) * shared[t]`` when a shared expert's result [n, D] and its gate's 32-bit
+    pre-activation (one number a token: a column of some matrix will do) are given.  Returns [n, D] of x's dtype."""
+    _gpu(mid, w_down, ids, weights, x, shared, shared_gate)
+    E = w_down.shape[0] if w_down.dim() == 3 else -1
+    _pairs(x, ids, E)
+    n, D = x.shape
+    top = ids.shape[1]
+    if w_down.dim() != 3 or w_down.shape[1] != D or w_down.dtype != x.dtype or not w_down.is_contiguous():
+        raise KernelError(f"expert_down_pairs: weights must be contiguous [E, {D}, F] of x's dtype")
+    F = w_down.shape[2]
+    if tuple(mid.shape) != (n, top, F) or mid.dtype != x.dtype or not mid.is_contiguous():
+        raise KernelError(f"expert_down_pairs: mid must be contiguous [{n}, {top}, {F}] of x's dtype")
+    if tuple(weights.shape) != (n, top) or weights.dtype != torch.float32 or not weights.is_contiguous():
+        raise KernelError("expert_down_pairs: weights must be contiguous float32 [n, top]")
+    sg_stride = 0
+    if shared is not None:
+        if tuple(shared.shape) != (n, D) or shared.dtype != x.dtype or not shared.is_contiguous():
+            raise KernelError("expert_down_pairs: the shared expert's result must be contiguous [n, D] of x's dtype")
+        if shared_gate is None or shared_gate.dtype != torch.float32 or shared_gate.numel() != n or shared_gate.dim() > 2:
+            raise KernelError("expert_down_pairs: the shared expert's gate must be float32, one number a token")
+        sg_stride = shared_gate.stride(0) if n > 1 else 1
+    out = torch.empty((n, D), dtype=x.dtype, device=x.device)
+    check(core().tl_expert_down_pairs(mid.data_ptr(), w_down.data_ptr(), ids.data_ptr(), weights.data_ptr(), top, E, x.data_ptr(),
+                                      _ptr(shared), _ptr(shared_gate), sg_stride, out.data_ptr(), n, D, F, dtype_code(x.dtype),
+                                      _stream()))
+    return out
+
+
+def bias_gelu_(x: torch.Tensor, bias: torch.Tensor) -> torch.Tensor:
+    """``x <- gelu(x + bias)`` in place, row by row, with the exact gelu ``z/2 (1 + erf(z / sqrt 2))`` in 32-bit."""
+    _gpu(x, bias)
+    if x.dim() != 2 or not x.is_contiguous():
+        raise KernelError("bias_gelu_: x must be a contiguous matrix")
+    if tuple(bias.shape) != (x.shape[1],) or bias.dtype != x.dtype or not bias.is_contiguous():
+        raise KernelError(f"bias_gelu_: bias must be a contiguous vector of {x.shape[1]} entries of x's dtype")
+    check(core().tl_bias_gelu(x.data_ptr(), bias.data_ptr(), x.shape[0], x.shape[1], dtype_code(x.dtype), _stream()))
+    return x
+
+
+def weighted_pair(a: torch.Tensor, a_scale: float, b: torch.Tensor, b_scale: float) -> torch.Tensor:
+    """``a_scale * a + b_scale * b`` in 32-bit, rounded once to the tensors' dtype."""
+    _gpu(a, b)
+    if a.shape != b.shape or a.dtype != b.dtype or not a.is_contiguous() or not b.is_contiguous():
+        raise KernelError("weighted_pair: two contiguous tensors of one shape and dtype")
+    out = torch.empty_like(a)
+    check(core().tl_weighted_pair(a.data_ptr(), float(a_scale), b.data_ptr(), float(b_scale), out.data_ptr(), a.numel(),
+                                  dtype_code(a.dtype), _stream()))
+    return out
+
+
+def post_norm_add_norm(
+    stream: torch.Tensor,
+    branch: torch.Tensor,
+    post_weight: torch.Tensor,
+    eps: float,
+    next_weight: Optional[torch.Tensor] = None,
+    next_eps: float = 0.0,
+) -> Optional[torch.Tensor]:
+    """``stream += branch / rms(branch) * post_weight`` in place and in 32-bit, and, with ``next_weight``, the rows
+    ``stream / rms(stream) * next_weight`` in the branch's dtype: the norm behind a branch and the norm before the next
+    one, one pass over each row.  Both weights are 32-bit vectors (whatever factors a norm has, folded into one)."""
+    _gpu(stream, branch, post_weight, next_weight)
+    if stream.dim() != 2 or stream.dtype != torch.float32 or not stream.is_contiguous():
+        raise KernelError("post_norm_add_norm: the stream must be a contiguous float32 matrix")
+    n, hidden = stream.shape
+    if tuple(branch.shape) != (n, hidden) or not branch.is_contiguous():
+        raise KernelError("post_norm_add_norm: the branch must be contiguous and of the stream's shape")
+    for w in (post_weight, next_weight):
+        if w is not None and (tuple(w.shape) != (hidden,) or w.dtype != torch.float32 or not w.is_contiguous()):
+            raise KernelError(f"post_norm_add_norm: weights must be float32 vectors of {hidden} entries")
+    rows = torch.empty_like(branch) if next_weight is not None else None
+    check(core().tl_post_norm_add_norm(stream.data_ptr(), branch.data_ptr(), post_weight.data_ptr(), float(eps), _ptr(next_weight),
+                                       float(next_eps), _ptr(rows), n, hidden, dtype_code(branch.dtype), _stream()))
+    return rows

@@ -306,6 +306,9 @@ def gated_delta(
     n_key_heads: int,
     head_dim: int,
     v_head_dim: int,
+    gate: Optional[torch.Tensor] = None,
+    gate_act: str = "silu",
+    channel_decay: Optional[torch.Tensor] = None,
 ) -> torch.Tensor:
     """The gated delta rule over each request's tokens, in 32-bit.  ``qkv`` [n, 2 G dk + H dv]: query
     heads | key heads | value heads, already convolved and activated.  Of ``proj`` [n, ..] the output
@@ -313,17 +316,31 @@ def gated_delta(
     decay (H columns each from ``b_offset`` and ``a_offset``) are read.  Per head, with unit q and k
     (q also times dk^-1/2): ``S <- decay S; u = beta (v - S^T k); S <- S + k u^T; o = S^T q``; then o
     over its root mean square, times ``norm_weight`` [dv], times silu(gate).  ``S`` lives at
-    ``state_offset`` of the request's state row, H * dv * dk floats.  Returns [n, H * dv]."""
-    _gpu(qkv, proj, A_log, dt_bias, norm_weight)
+    ``state_offset`` of the request's state row, H * dv * dk floats.  Returns [n, H * dv].
+
+    ``gate``: a matrix of its own that holds the output gate's columns from ``gate_offset`` (None: ``proj``);
+    ``gate_act`` "sigmoid": the gate is the logistic function of them, not silu.  ``channel_decay`` float32
+    [n, H * dk]: every key channel of a head (row of S) has a decay of its own,
+    ``exp(-exp(A_log[h]) softplus(channel_decay[t, h, i] + dt_bias[h, i]))`` with ``dt_bias`` of H * dk entries;
+    the column ``a_offset`` of ``proj`` is then not read."""
+    _gpu(qkv, proj, A_log, dt_bias, norm_weight, gate, channel_decay)
     H, G, dk, dv = n_heads, n_key_heads, head_dim, v_head_dim
     n = qkv.shape[0]
+    if gate_act not in ("silu", "sigmoid"):
+        raise KernelError(f"gated_delta: gate_act {gate_act!r} (silu, sigmoid)")
+    gate_src = proj if gate is None else gate
+    if gate_src.dim() != 2 or gate_src.shape[0] != n or gate_src.stride(1) != 1 or gate_src.dtype != qkv.dtype:
+        raise KernelError("gated_delta: the gate must be a matrix of qkv's dtype with a row per token")
+    if channel_decay is not None and (channel_decay.dim() != 2 or tuple(channel_decay.shape) != (n, H * dk)
+                                      or channel_decay.dtype != torch.float32 or channel_decay.stride(1) != 1):
+        raise KernelError(f"gated_delta: channel_decay must be float32 [n, {H * dk}] with contiguous rows")
     if qkv.dim() != 2 or qkv.shape[1] != 2 * G * dk + H * dv or qkv.stride(1) != 1:
         raise KernelError(f"gated_delta: qkv must be [n, {2 * G * dk + H * dv}] with contiguous rows")
     if proj.dim() != 2 or proj.shape[0] != n or proj.stride(1) != 1 or proj.dtype != qkv.dtype:
         raise KernelError("gated_delta: proj must be a matrix of qkv's dtype with a row per token")
-    if gate_offset + H * dv > proj.shape[1] or max(b_offset, a_offset) + H > proj.shape[1]:
+    if gate_offset + H * dv > gate_src.shape[1] or (b_offset if channel_decay is not None else max(b_offset, a_offset)) + H > proj.shape[1]:
         raise KernelError("gated_delta: gate, b or a do not lie in the rows of proj")
-    for v, size in ((A_log, H), (dt_bias, H), (norm_weight, dv)):
+    for v, size in ((A_log, H), (dt_bias, H if channel_decay is None else H * dk), (norm_weight, dv)):
         if tuple(v.shape) != (size,) or v.dtype != torch.float32 or not v.is_contiguous():
             raise KernelError(f"gated_delta: a float32 vector of {size} entries expected, got {tuple(v.shape)} {v.dtype}")
     n_seqs = _step_rows(None, qo_indptr, slot_ids, n, state)
@@ -334,7 +351,75 @@ def gated_delta(
         core().tl_gated_delta(
             qkv.data_ptr(), qkv.stride(0), proj.data_ptr(), proj.stride(0), gate_offset, b_offset, a_offset, A_log.data_ptr(),
             dt_bias.data_ptr(), norm_weight.data_ptr(), float(eps), region, stride, qo_indptr.data_ptr(), slot_ids.data_ptr(),
-            out.data_ptr(), n, n_seqs, H, G, dk, dv, o_raw.data_ptr(), dtype_code(qkv.dtype), _stream(),
+            out.data_ptr(), n, n_seqs, H, G, dk, dv, o_raw.data_ptr(), dtype_code(qkv.dtype), gate_src.data_ptr(), gate_src.stride(0),
+            1 if gate_act == "sigmoid" else 0, _ptr(channel_decay), channel_decay.stride(0) if channel_decay is not None else 0,
+            _stream(),
+        )
+    )
+    return out
+
+
+def matrix_memory_state_size(n_heads: int, head_dim: int, v_head_dim: int) -> int:
+    """32-bit elements of a request's state row that ``matrix_memory`` keeps: per head the matrix and the normaliser
+    as dv + 1 columns of dk, and the running maximum once for every column."""
+    return n_heads * (v_head_dim + 1) * head_dim + n_heads * (v_head_dim + 1)
+
+
+def matrix_memory(
+    proj: torch.Tensor,
+    q_offset: int,
+    k_offset: int,
+    v_offset: int,
+    i_offset: int,
+    f_offset: int,
+    gate_offset: int,
+    i_bias: torch.Tensor,
+    f_bias: torch.Tensor,
+    gate_cap: float,
+    norm_weight: torch.Tensor,
+    eps: float,
+    state: torch.Tensor,
+    state_offset: int,
+    qo_indptr: torch.Tensor,
+    slot_ids: torch.Tensor,
+    n_heads: int,
+    head_dim: int,
+    v_head_dim: int,
+) -> torch.Tensor:
+    """The matrix memory of an mLSTM layer over each request's tokens, in 32-bit.  Of ``proj`` [n, ..] the columns of
+    q and k (H heads of dk each), v and the output gate (H heads of dv) and the pre-activations of the input and the
+    forget gate (H each) are read from their offsets.  Per head, with ``i = cap tanh((i~ + i_bias) / cap)`` and
+    ``f = logsigmoid(cap tanh((f~ + f_bias) / cap))`` and a running maximum m (0 at the start):
+    ``m' = max(f + m, i); C <- exp(f + m - m') C + exp(i - m') k v^T``, n likewise with k alone,
+    ``o = C^T q dk^-1/2 / (max(|n . q dk^-1/2|, exp(-m')) + 1e-6)``; then o over its root mean square, times
+    ``norm_weight`` [H * dv], times sigmoid(gate).  C, n and m live at ``state_offset`` of the request's state row
+    (``matrix_memory_state_size`` floats).  Returns [n, H * dv]."""
+    _gpu(proj, i_bias, f_bias, norm_weight)
+    H, dk, dv = n_heads, head_dim, v_head_dim
+    n = proj.shape[0]
+    if proj.dim() != 2 or proj.stride(1) != 1:
+        raise KernelError("matrix_memory: proj must be a matrix with contiguous rows")
+    width = proj.shape[1]
+    for off, size, what in ((q_offset, H * dk, "q"), (k_offset, H * dk, "k"), (v_offset, H * dv, "v"), (gate_offset, H * dv, "gate"),
+                            (i_offset, H, "i"), (f_offset, H, "f")):
+        if off < 0 or off + size > width:
+            raise KernelError(f"matrix_memory: the columns of {what} do not lie in the rows of proj")
+    for v, size in ((i_bias, H), (f_bias, H), (norm_weight, H * dv)):
+        if tuple(v.shape) != (size,) or v.dtype != torch.float32 or not v.is_contiguous():
+            raise KernelError(f"matrix_memory: a float32 vector of {size} entries expected, got {tuple(v.shape)} {v.dtype}")
+    if not gate_cap > 0:
+        raise KernelError("matrix_memory: the gates' cap must be positive")
+    n_seqs = _step_rows(None, qo_indptr, slot_ids, n, state)
+    region, stride = state_region(state, state_offset, matrix_memory_state_size(H, dk, dv))
+    out = torch.empty((n, H * dv), dtype=proj.dtype, device=proj.device)
+    o_raw = torch.empty((n, H * dv), dtype=torch.float32, device=proj.device)
+    den = torch.empty((n, H), dtype=torch.float32, device=proj.device)
+    check(
+        core().tl_matrix_memory(
+            proj.data_ptr(), proj.stride(0), q_offset, k_offset, v_offset, i_offset, f_offset, i_bias.data_ptr(), f_bias.data_ptr(),
+            float(gate_cap), proj.data_ptr(), proj.stride(0), gate_offset, norm_weight.data_ptr(), float(eps), region, stride,
+            qo_indptr.data_ptr(), slot_ids.data_ptr(), out.data_ptr(), n, n_seqs, H, dk, dv, o_raw.data_ptr(), den.data_ptr(),
+            dtype_code(proj.dtype), _stream(),
         )
     )
     return out

@@ -42,6 +42,9 @@ class Attention(Mixer):
     "mix" turns its values into ``(1 - m) v + m v_source`` of the same token before they are cached (``m``: the
     tensor ``vmix``, one number); ``out_gate``: the heads' outputs are multiplied by the sigmoid of a projection of
     the layer's input (tensor ``wg.weight``), "channel" by channel or "head" by head.
+
+    ``values_from_keys``: there is no value projection; a token's values are its keys as projected, before the
+    rotation (the key rows of the fused projection stand in it a second time as value rows).
     """
 
     #: every launch is fixed by the step's shape: a decode step may be recorded in a HIP graph
@@ -71,7 +74,11 @@ class Attention(Mixer):
         value_mix: Optional[str] = None,
         value_mix_key: str = "values",
         out_gate: Optional[str] = None,
+        values_from_keys: bool = False,
     ):
+        self.values_from_keys = bool(values_from_keys)
+        if self.values_from_keys and (shares_kv or (v_head_dim and v_head_dim != head_dim) or qkv_bias):
+            raise ValueError("attention: values that are the keys have the keys' head size, no bias, and a cache of their own")
         if num_heads % num_kv_heads:
             raise ValueError(f"{num_heads} heads are not a multiple of {num_kv_heads} kv heads")
         self.hidden_size = hidden_size
@@ -136,7 +143,8 @@ class Attention(Mixer):
                  "wo.weight": ParamSpec((self.hidden_size, self.num_heads * self.v_head_dim))}
         if not self.shares_kv:
             specs["wk.weight"] = ParamSpec((kv, self.hidden_size))
-            specs["wv.weight"] = ParamSpec((self.num_kv_heads * self.v_head_dim, self.hidden_size))
+            if not self.values_from_keys:
+                specs["wv.weight"] = ParamSpec((self.num_kv_heads * self.v_head_dim, self.hidden_size))
         if self.has_sinks:
             specs["sinks"] = ParamSpec((self.num_heads,), kind="vector", init="zeros")
         if self.qkv_bias:
@@ -189,7 +197,7 @@ class Attention(Mixer):
                       v_head_dim=self.v_head_dim if self.v_head_dim != self.head_dim else None)
 
     def bind(self, tensors: Dict[str, torch.Tensor]) -> None:
-        names = ["wq"] if self.shares_kv else ["wq", "wk", "wv"]
+        names = ["wq"] if self.shares_kv else ["wq", "wk", "wk" if self.values_from_keys else "wv"]
         # one fused projection [q rows | k rows | v rows | gate rows]: a single matrix product per token batch
         self.wqkv = torch.cat([tensors[f"{n}.weight"] for n in names + (["wg"] if self.out_gate else [])], dim=0).contiguous()
         if self.qk_norm_weight:

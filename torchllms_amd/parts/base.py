@@ -226,6 +226,11 @@ class Block(Part):
             prefix = slot + "."
             part.bind({k[len(prefix):]: v for k, v in tensors.items() if k.startswith(prefix)})
 
+    def expects(self, following: Optional["Block"]) -> None:
+        """Told once, when the model is put together: the arrangement that runs right after this one in every run of
+        this layer (None: the last layer, or a layer whose runs are followed by different arrangements).  An
+        arrangement may leave work to, or do work for, the one that follows; the default does neither."""
+
     def forward(self, h, delta, ctx, cache):
         raise NotImplementedError
 

@@ -117,3 +117,97 @@ class BranchNormMixerBlock(_BranchNorm):
         h, x = self.norm1.forward_branch(h, self.mix.forward(self.rows_of(h, ctx), ctx, cache["mix"]))
         self.keep_rows(h, x, ctx)
         return h, None
+
+
+class _Sandwich(Block):
+    """Layers with a norm before and a norm behind every branch, over a 32-bit residual stream:
+    ``x <- x + post(branch(pre(x)))``, one branch after the other.  The norm behind a branch and the norm before the
+    next one (of this layer or of the next layer of this kind) run as one kernel over the rows: a layer hands the
+    rows that the next layer's first norm would make on, under ``_ROWS`` of the step's scratch, when the next layer
+    has said (``expects``) which norm that is."""
+
+    graph_safe = True
+    _ROWS = "sandwich_rows"  # in ctx.scratch: (the stream the rows were made from, the norm that made them, the rows)
+
+    def first_norm(self):
+        return self.norm1
+
+    def __init__(self, parts):
+        super().__init__(parts)
+        self.next_first_norm = None  # the first norm of the layer that runs after this one, if that is known
+
+    def expects(self, following: "Block") -> None:
+        """Told once, when the model is put together: ``following`` runs right after this layer."""
+        self.next_first_norm = following.first_norm() if isinstance(following, _Sandwich) else None
+
+    def rows_for(self, norm, h, ctx):
+        kept = ctx.scratch.get(self._ROWS)
+        if kept is not None and kept[0] is h and kept[1] is norm:
+            return kept[2]
+        return norm.forward(h)
+
+    def mix_branch(self, y, ctx, cache):
+        raise NotImplementedError
+
+    def forward(self, h, delta, ctx, cache):
+        if delta is not None:
+            h = h + ops.resolved(delta).float()
+        a = self.mix_branch(self.rows_for(self.norm1, h, ctx), ctx, cache)
+        has_mlp = "mlp" in self.parts
+        after = self.norm2 if has_mlp else self.next_first_norm
+        h, y = self.norm1b.forward_branch_then(h, a, after)
+        if has_mlp:
+            after = self.next_first_norm
+            h, y = self.norm2b.forward_branch_then(h, self.mlp.forward(y, ctx), after)
+        if after is not None:
+            ctx.scratch[self._ROWS] = (h, after, y)
+        return h, None
+
+
+@BLOCKS.register("sandwich")
+class SandwichBlock(_Sandwich):
+    """``x <- x + norm1b(mix(norm1(x))); x <- x + norm2b(mlp(norm2(x)))``."""
+
+    SLOTS = {"norm1": "norm", "mix": "mixer", "norm1b": "norm", "norm2": "norm", "mlp": "feed_forward", "norm2b": "norm"}
+
+    def mix_branch(self, y, ctx, cache):
+        return self.mix.forward(y, ctx, cache["mix"])
+
+
+@BLOCKS.register("sandwich_mixer")
+class SandwichMixerBlock(_Sandwich):
+    """The same layer without a feed-forward: ``x <- x + norm1b(mix(norm1(x)))``."""
+
+    SLOTS = {"norm1": "norm", "mix": "mixer", "norm1b": "norm"}
+
+    def mix_branch(self, y, ctx, cache):
+        return self.mix.forward(y, ctx, cache["mix"])
+
+
+class _SandwichPair(_Sandwich):
+    """Two mixers side by side that read the same normed rows; the branch is
+    ``left_scale * left(h) + right_scale * right(h)``.  Each keeps a cache entry of its own."""
+
+    def __init__(self, parts, left_scale: float = 1.0, right_scale: float = 1.0):
+        super().__init__(parts)
+        self.left_scale, self.right_scale = float(left_scale), float(right_scale)
+
+    def mix_branch(self, y, ctx, cache):
+        a = ops.resolved(self.left.forward(y, ctx, cache["left"]))
+        b = ops.resolved(self.right.forward(y, ctx, cache["right"]))
+        return ops.weighted_pair(a, self.left_scale, b, self.right_scale)
+
+
+@BLOCKS.register("sandwich_pair")
+class SandwichPairBlock(_SandwichPair):
+    """``x <- x + norm1b(s_l left(norm1(x)) + s_r right(norm1(x))); x <- x + norm2b(mlp(norm2(x)))``."""
+
+    SLOTS = {"norm1": "norm", "left": "mixer", "right": "mixer", "norm1b": "norm", "norm2": "norm", "mlp": "feed_forward",
+             "norm2b": "norm"}
+
+
+@BLOCKS.register("sandwich_pair_mixer")
+class SandwichPairMixerBlock(_SandwichPair):
+    """The same layer without a feed-forward."""
+
+    SLOTS = {"norm1": "norm", "left": "mixer", "right": "mixer", "norm1b": "norm"}

@@ -41,3 +41,102 @@ class SwiGLU(FeedForward):
 
     def forward(self, x, ctx):
         return ops.linear_to_sum(ops.linear_glu(x, self.w13, self.activation), self.w2, may_wait=True)
+
+
+@FEED_FORWARDS.register("dense_gelu")
+class DenseGelu(FeedForward):
+    """``W_down gelu(W_up x + b_up) + b_down`` with the exact gelu ``z/2 (1 + erf(z / sqrt 2))``."""
+
+    graph_safe = True
+
+    def __init__(self, hidden_size: int, intermediate_size: int):
+        self.hidden_size, self.intermediate_size = hidden_size, intermediate_size
+        self.w_up = self.b_up = self.w_down = self.b_down = None
+
+    def param_specs(self) -> Dict[str, ParamSpec]:
+        f, d = self.intermediate_size, self.hidden_size
+        return {"up.weight": ParamSpec((f, d)), "up.bias": ParamSpec((f,), init="zeros"),
+                "down.weight": ParamSpec((d, f)), "down.bias": ParamSpec((d,), init="zeros")}
+
+    def bind(self, tensors: Dict[str, torch.Tensor]) -> None:
+        self.w_up, self.w_down = tensors["up.weight"].contiguous(), tensors["down.weight"].contiguous()
+        self.b_up, self.b_down = tensors["up.bias"].contiguous(), tensors["down.bias"].contiguous()
+
+    def linear_weights(self):
+        return [self.w_up, self.w_down]
+
+    def forward(self, x, ctx):
+        mid = ops.bias_gelu_(ops.linear(ops.resolved(x), self.w_up), self.b_up)
+        return ops.add_bias_(ops.linear(mid, self.w_down), self.b_down)
+
+
+@FEED_FORWARDS.register("routed")
+class RoutedExperts(FeedForward):
+    """A mixture of ``num_experts`` gated feed-forwards ``W_down (silu(W_gate x) * (W_up x))`` without biases, of which
+    every token uses ``top``.  The router's outputs ``z = W_router x`` (32-bit) number ``num_experts + num_identity``;
+    the last ``num_identity`` stand for experts that hand their input through.  Scores ``s = softmax(z)`` over all
+    outputs; the ``top`` outputs with the largest ``s + correction`` are chosen, and the result is the sum of the
+    chosen experts' outputs times their ``s`` (not renormalised).  ``shared_size`` f > 0: an expert of that width runs
+    for every token and is added times ``sigmoid(W_sg x)``, one number a token.
+
+    A token's result depends on nothing but the token.  Every (token, choice) is worked on by itself, whatever the
+    step's shape, so a decode step's launches are fixed by its shape."""
+
+    graph_safe = True
+
+    def __init__(self, hidden_size: int, expert_size: int, num_experts: int, top: int, num_identity: int = 0, shared_size: int = 0):
+        for name, v in (("expert_size", expert_size), ("num_experts", num_experts), ("top", top)):
+            if not isinstance(v, int) or v <= 0:
+                raise ValueError(f"routed: {name} must be a positive integer, got {v!r}")
+        if num_identity < 0 or shared_size < 0 or top > num_experts + num_identity:
+            raise ValueError(f"routed: {top} choices among {num_experts} + {num_identity} outputs; sizes must not be negative")
+        self.hidden_size, self.F, self.E, self.I, self.top, self.shared = hidden_size, expert_size, num_experts, num_identity, top, shared_size
+        self.w_router = self.correction = self.w_gu = self.w_down = self.shared_w13 = self.shared_w2 = None
+
+    def param_specs(self) -> Dict[str, ParamSpec]:
+        d, f, n = self.hidden_size, self.F, self.E + self.I
+        specs = {"router.weight": ParamSpec((n, d), init="wide"), "correction": ParamSpec((n,), init="zeros")}
+        for e in range(self.E):
+            specs[f"experts.{e}.w1.weight"] = ParamSpec((f, d))
+            specs[f"experts.{e}.w3.weight"] = ParamSpec((f, d))
+            specs[f"experts.{e}.w2.weight"] = ParamSpec((d, f))
+        if self.shared:
+            specs["shared.w1.weight"] = ParamSpec((self.shared, d))
+            specs["shared.w3.weight"] = ParamSpec((self.shared, d))
+            specs["shared.w2.weight"] = ParamSpec((d, self.shared))
+            specs["shared.gate.weight"] = ParamSpec((1, d))
+        return specs
+
+    def check_sizes(self, dtype: torch.dtype) -> None:
+        if self.E + self.I > ops.ROUTER_MAX_OUTPUTS:
+            raise ValueError(f"routed: a router of {self.E + self.I} outputs; the kernel takes up to {ops.ROUTER_MAX_OUTPUTS}")
+        lds = ops.device_facts()[1]
+        if 4 * max(self.hidden_size, self.top * self.F) > lds:
+            raise ValueError(f"routed: rows of {self.hidden_size} elements or {self.top} choices of {self.F} do not fit {lds} bytes of LDS")
+
+    def bind(self, tensors: Dict[str, torch.Tensor]) -> None:
+        # the router's matrix, and under it the shared expert's gate: one product with 32-bit results
+        rows = [tensors["router.weight"]] + ([tensors["shared.gate.weight"]] if self.shared else [])
+        self.w_router = torch.cat(rows, dim=0).contiguous()
+        self.correction = tensors["correction"].float().contiguous()
+        self.w_gu = torch.stack([torch.cat([tensors[f"experts.{e}.w1.weight"], tensors[f"experts.{e}.w3.weight"]], dim=0)
+                                 for e in range(self.E)]).contiguous()
+        self.w_down = torch.stack([tensors[f"experts.{e}.w2.weight"] for e in range(self.E)]).contiguous()
+        if self.shared:
+            self.shared_w13 = torch.cat([tensors["shared.w1.weight"], tensors["shared.w3.weight"]], dim=0).contiguous()
+            self.shared_w2 = tensors["shared.w2.weight"].contiguous()
+
+    def linear_weights(self):
+        return [(self.w_router, "plain", torch.float32), (self.shared_w13, "glu"), self.shared_w2]
+
+    def forward(self, x, ctx):
+        x = ops.resolved(x)
+        n_out = self.E + self.I
+        z = ops.linear(x, self.w_router, out_dtype=torch.float32)
+        ids, weights = ops.router_topk(z, n_out, self.correction, self.top)
+        mid = ops.expert_glu_pairs(x, self.w_gu, ids)
+        shared = gate = None
+        if self.shared:
+            shared = ops.linear(ops.linear_glu(x, self.shared_w13), self.shared_w2)
+            gate = z[:, n_out]
+        return ops.expert_down_pairs(mid, self.w_down, ids, weights, x, shared, gate)

@@ -48,6 +48,14 @@ class Model:
             self.blocks.append(block_cls(parts, **layer.block_params))
         self.final_norm = NORMS.build(spec.final_norm)
         self.head = HEADS.build(spec.head)
+        # every arrangement learns which one follows it, where that is the same in all of its runs
+        followers: Dict[int, set] = {}
+        for pos, run in enumerate(spec.order):
+            nxt = spec.order[pos + 1].layer if pos + 1 < len(spec.order) else None
+            followers.setdefault(run.layer, set()).add(nxt)
+        for layer, nexts in followers.items():
+            only = next(iter(nexts)) if len(nexts) == 1 else None
+            self.blocks[layer].expects(self.blocks[only] if only is not None else None)
         # per run: (slot of a mixer, key of its cache entry, whether the run owns the entry)
         self._run_caches: List[List[Tuple[str, Tuple[int, str], bool]]] = []
         for run_id, run in enumerate(spec.order):

@@ -18,24 +18,38 @@ class RMSNorm(Norm):
     ``stream_dtype`` "float32": the norm works beside a 32-bit residual stream whatever the model's dtype.
     Then ``y = cast(x32 * rsqrt(mean(x32^2) + eps) * weight32)``, rounded once; it reads rows of the stream or of
     the model's dtype and hands on rows of the model's dtype, and ``forward_branch`` adds a normed branch to the
-    stream (``stream += norm(branch)``), which is what a block that norms its branches' outputs calls."""
+    stream (``stream += norm(branch)``), which is what a block that norms its branches' outputs calls.
+
+    Beside a 32-bit stream the weight may be stored around another number than one (``offset`` c: the factor is
+    ``c + weight``) and a second vector may follow it (``scaled``: the tensor ``scale``, a layer's scale on a normed
+    branch): ``y = x32 * rsqrt(mean(x32^2) + eps) * (c + weight32) * scale32``.  Both are folded into one 32-bit
+    vector when the tensors arrive (``factor``).  ``forward_branch_then`` adds a normed branch to the stream and
+    hands on what another norm makes of the new stream, in one pass."""
 
     graph_safe = True
     takes_split_sums = True  # ops.rmsnorm adds the slices of a split product while it reads them
 
-    def __init__(self, size: int, eps: float, stream_dtype: Optional[str] = None):
+    def __init__(self, size: int, eps: float, stream_dtype: Optional[str] = None, offset: float = 0.0, scaled: bool = False):
         if stream_dtype not in (None, "float32"):
             raise ValueError(f"rmsnorm: stream_dtype {stream_dtype!r} (None: the model's dtype, or \"float32\")")
+        if stream_dtype is None and (float(offset) != 0.0 or scaled):
+            raise ValueError("rmsnorm: an offset of the weight or a second scale needs the 32-bit residual stream (stream_dtype=\"float32\")")
         self.size = size
         self.eps = float(eps)
         self.stream_dtype = stream_dtype
+        self.offset = float(offset)
+        self.scaled = bool(scaled)
         self.takes_split_sums = stream_dtype is None
         self.weight: Optional[torch.Tensor] = None
         self.out_dtype: Optional[torch.dtype] = None
 
     def param_specs(self) -> Dict[str, ParamSpec]:
         # (beside a 32-bit stream the vector follows the model's dtype, which is the dtype of the normed rows)
-        return {"weight": ParamSpec((self.size,), kind="vector" if self.stream_dtype is None else "matrix", init="ones")}
+        specs = {"weight": ParamSpec((self.size,), kind="vector" if self.stream_dtype is None else "matrix",
+                                     init="ones" if self.offset == 0.0 else "normal")}
+        if self.scaled:
+            specs["scale"] = ParamSpec((self.size,), kind="matrix", init="fraction")
+        return specs
 
     def check_sizes(self, dtype: torch.dtype) -> None:
         if not 0 < self.size <= ops.rmsnorm_max_hidden():
@@ -45,7 +59,26 @@ class RMSNorm(Norm):
         self.weight = tensors["weight"].contiguous()
         if self.stream_dtype is not None:
             self.out_dtype = self.weight.dtype
-            self.weight = self.weight.float().contiguous()
+            self.weight = self.weight.float()
+            if self.offset != 0.0:
+                self.weight = self.weight + self.offset
+            if self.scaled:
+                self.weight = self.weight * tensors["scale"].float()
+            self.weight = self.weight.contiguous()
+
+    @property
+    def factor(self) -> torch.Tensor:
+        """Beside a 32-bit stream: the 32-bit vector a normed row is multiplied by (offset and scale folded in)."""
+        return self.weight
+
+    def forward_branch_then(self, stream: torch.Tensor, branch, then: Optional["RMSNorm"]):
+        """``stream += norm(branch)`` in place, and ``then.forward(stream)`` of the new stream from the same pass
+        over the rows (None when ``then`` is None: nobody reads them).  Returns ``(stream, rows)``."""
+        if self.stream_dtype is None or (then is not None and (not isinstance(then, RMSNorm) or then.stream_dtype is None)):
+            raise ValueError("rmsnorm: forward_branch_then joins two RMS norms beside the 32-bit residual stream")
+        rows = ops.post_norm_add_norm(stream, ops.resolved(branch), self.weight, self.eps,
+                                      then.weight if then is not None else None, then.eps if then is not None else 0.0)
+        return stream, rows
 
     def forward(self, x: torch.Tensor) -> torch.Tensor:
         if self.stream_dtype is not None:

@@ -99,17 +99,32 @@ class GatedDelta(Mixer):
     ``decay = exp(-exp(A_log) softplus(W_a h + dt_bias))`` per head.  Per head and token
     ``S <- decay S; u = beta (v - S^T k); S <- S + k u^T; o = S^T q``; o is divided by its root mean
     square over v_head_dim, multiplied by the weight ``norm`` and by ``silu(W_g h)``, then projected by
-    W_o.  Gates, decays, unit norms and the state are 32-bit."""
+    W_o.  Gates, decays, unit norms and the state are 32-bit.
+
+    ``decay`` "channel": every key channel of a head (row of S) has a decay of its own,
+    ``exp(-exp(A_log_h) softplus(a_{h,i} + dt_bias_{h,i}))``, whose pre-activation comes through two matrices,
+    ``a = W_a2 (W_a1 h)`` with ``decay_rank`` numbers in between (tensors ``a1``, ``a2``; 32-bit results).
+    ``gate_rank`` r: the output gate comes through two matrices as well, ``W_g2 (W_g1 h)`` (tensors ``g1``, ``g2``).
+    ``gate_act`` "sigmoid": the gate is the logistic function of its pre-activation instead of silu."""
 
     graph_safe = True
 
     def __init__(self, hidden_size: int, num_heads: int, num_key_heads: int, head_dim: int, v_head_dim: int, conv_taps: int,
-                 norm_eps: float):
+                 norm_eps: float, decay: str = "head", decay_rank: Optional[int] = None, gate_rank: Optional[int] = None,
+                 gate_act: str = "silu"):
         if num_heads % num_key_heads:
             raise ValueError(f"gated_delta: {num_heads} heads are not a multiple of {num_key_heads} key heads")
+        if decay not in ("head", "channel") or gate_act not in ("silu", "sigmoid"):
+            raise ValueError("gated_delta: decay is \"head\" or \"channel\", gate_act \"silu\" or \"sigmoid\"")
+        if (decay == "channel") != (decay_rank is not None):
+            raise ValueError("gated_delta: a decay per channel comes through two matrices (decay_rank), a decay per head through one")
+        for name, v in (("decay_rank", decay_rank), ("gate_rank", gate_rank)):
+            if v is not None and (not isinstance(v, int) or v <= 0):
+                raise ValueError(f"gated_delta: {name} must be a positive integer, got {v!r}")
         self.hidden_size, self.H, self.G, self.dk, self.dv, self.taps = hidden_size, num_heads, num_key_heads, head_dim, v_head_dim, conv_taps
         self.norm_eps = float(norm_eps)
-        self.w_all = self.w_o = self.conv_w = self.A_log = self.dt_bias = self.norm_w = None
+        self.decay, self.decay_rank, self.gate_rank, self.gate_act = decay, decay_rank, gate_rank, gate_act
+        self.w_all = self.w_o = self.conv_w = self.A_log = self.dt_bias = self.norm_w = self.w_a2 = self.w_g2 = None
 
     @property
     def conv_channels(self) -> int:
@@ -117,15 +132,28 @@ class GatedDelta(Mixer):
 
     def param_specs(self) -> Dict[str, ParamSpec]:
         d, qk, v = self.hidden_size, self.G * self.dk, self.H * self.dv
-        return {
+        specs = {
             "q": ParamSpec((qk, d)), "q.conv": ParamSpec((qk, self.taps), init="conv"),
             "k": ParamSpec((qk, d)), "k.conv": ParamSpec((qk, self.taps), init="conv"),
             "v": ParamSpec((v, d)), "v.conv": ParamSpec((v, self.taps), init="conv"),
-            "b": ParamSpec((self.H, d)), "a": ParamSpec((self.H, d)),
-            "A_log": ParamSpec((self.H,), init="zeros"), "dt_bias": ParamSpec((self.H,), init="zeros"),
+            "b": ParamSpec((self.H, d)),
+            "A_log": ParamSpec((self.H,), init="zeros"),
             "norm": ParamSpec((self.dv,), init="ones"),
-            "g": ParamSpec((v, d)), "o": ParamSpec((d, v)),
+            "o": ParamSpec((d, v)),
         }
+        if self.decay == "channel":
+            specs["a1"] = ParamSpec((self.decay_rank, d))
+            specs["a2"] = ParamSpec((self.H * self.dk, self.decay_rank), init="wide")
+            specs["dt_bias"] = ParamSpec((self.H * self.dk,), init="zeros")
+        else:
+            specs["a"] = ParamSpec((self.H, d))
+            specs["dt_bias"] = ParamSpec((self.H,), init="zeros")
+        if self.gate_rank is not None:
+            specs["g1"] = ParamSpec((self.gate_rank, d))
+            specs["g2"] = ParamSpec((v, self.gate_rank), init="wide")
+        else:
+            specs["g"] = ParamSpec((v, d))
+        return specs
 
     def check_sizes(self, dtype: torch.dtype) -> None:
         if self.dk > 256:
@@ -137,8 +165,12 @@ class GatedDelta(Mixer):
         return StateNeed(shape=((self.taps - 1) * self.conv_channels + self.H * self.dv * self.dk,), dtype="float32")
 
     def bind(self, tensors: Dict[str, torch.Tensor]) -> None:
-        # one projection [q | k | v | output gate | write strength | decay]: a single product per step
-        self.w_all = torch.cat([tensors[n] for n in ("q", "k", "v", "g", "b", "a")], dim=0).contiguous()
+        # one projection [q | k | v | output gate | write strength | decay]: a single product per step (of a gate or
+        # a decay that comes through two matrices, the first)
+        gate, decay = "g" if self.gate_rank is None else "g1", "a" if self.decay == "head" else "a1"
+        self.w_all = torch.cat([tensors[n] for n in ("q", "k", "v", gate, "b", decay)], dim=0).contiguous()
+        self.w_g2 = tensors["g2"].contiguous() if self.gate_rank is not None else None
+        self.w_a2 = tensors["a2"].contiguous() if self.decay == "channel" else None
         self.conv_w = torch.cat([tensors[n + ".conv"] for n in ("q", "k", "v")], dim=0).float().t().contiguous()  # [taps, channels]
         self.w_o = tensors["o"].contiguous()
         self.A_log = tensors["A_log"].float().contiguous()
@@ -146,13 +178,82 @@ class GatedDelta(Mixer):
         self.norm_w = tensors["norm"].float().contiguous()
 
     def linear_weights(self):
-        return [self.w_all, (self.w_o, "sum")]
+        return [self.w_all, (self.w_o, "sum"), self.w_g2, (self.w_a2, "plain", torch.float32)]
 
     def forward(self, x, ctx, cache):
-        c, hv = self.conv_channels, self.H * self.dv
+        c = self.conv_channels
+        g_cols = self.H * self.dv if self.gate_rank is None else self.gate_rank
+        b_at = c + g_cols
+        a_at = b_at + self.H
         state = cache.tensor
         proj = ops.linear(ops.resolved(x), self.w_all)
         qkv = ops.causal_conv(proj[:, :c], self.conv_w, None, state, 0, ctx.token_seq, ctx.qo_indptr, ctx.slot_ids)
-        y = ops.gated_delta(qkv, proj, c, c + hv, c + hv + self.H, self.A_log, self.dt_bias, self.norm_w, self.norm_eps, state,
-                            (self.taps - 1) * c, ctx.qo_indptr, ctx.slot_ids, self.H, self.G, self.dk, self.dv)
+        gate, gate_at = None, c
+        if self.gate_rank is not None:
+            gate, gate_at = ops.linear(proj[:, c:b_at], self.w_g2), 0
+        channel = None
+        if self.decay == "channel":
+            channel = ops.linear(proj[:, a_at : a_at + self.decay_rank], self.w_a2, out_dtype=torch.float32)
+        y = ops.gated_delta(qkv, proj, gate_at, b_at, a_at, self.A_log, self.dt_bias, self.norm_w, self.norm_eps, state,
+                            (self.taps - 1) * c, ctx.qo_indptr, ctx.slot_ids, self.H, self.G, self.dk, self.dv,
+                            gate=gate, gate_act=self.gate_act, channel_decay=channel)
+        return ops.linear_to_sum(y, self.w_o)
+
+
+@MIXERS.register("matrix_memory")
+class MatrixMemory(Mixer):
+    """The matrix memory of an mLSTM layer.  ``q`` (times head_dim^-1/2) and ``k`` (``num_heads`` heads of
+    ``head_dim``) and ``v`` (heads of ``v_head_dim``) are projections of the input, and so are, per head, the
+    pre-activations of a log input gate ``i = cap tanh((W_i h + b_i) / cap)`` and of a log forget gate
+    ``f = logsigmoid(cap tanh((W_f h + b_f) / cap))``.  Per head a matrix C, a vector n and a running maximum m
+    start at zero; for every token ``m' = max(f + m, i)``, ``C <- exp(f + m - m') C + exp(i - m') k v^T``, n likewise
+    with k alone, ``o = C^T q / (max(|n . q|, exp(-m')) + 1e-6)``.  Each head's o is divided by its root mean square,
+    the heads side by side are multiplied by the weight ``norm`` and by ``sigmoid(W_g h)``, then projected by W_o.
+    Gates, maxima, exponentials, the state and the norm are 32-bit."""
+
+    graph_safe = True
+
+    def __init__(self, hidden_size: int, num_heads: int, head_dim: int, v_head_dim: int, gate_cap: float, norm_eps: float):
+        for name, v in (("num_heads", num_heads), ("head_dim", head_dim), ("v_head_dim", v_head_dim)):
+            if not isinstance(v, int) or v <= 0:
+                raise ValueError(f"matrix_memory: {name} must be a positive integer, got {v!r}")
+        if not float(gate_cap) > 0:
+            raise ValueError(f"matrix_memory: gate_cap must be positive, got {gate_cap!r}")
+        self.hidden_size, self.H, self.dk, self.dv = hidden_size, num_heads, head_dim, v_head_dim
+        self.gate_cap, self.norm_eps = float(gate_cap), float(norm_eps)
+        self.w_all = self.w_o = self.i_b = self.f_b = self.norm_w = None
+
+    def param_specs(self) -> Dict[str, ParamSpec]:
+        d, qk, v = self.hidden_size, self.H * self.dk, self.H * self.dv
+        return {
+            "q": ParamSpec((qk, d)), "k": ParamSpec((qk, d)), "v": ParamSpec((v, d)), "g": ParamSpec((v, d)),
+            "i": ParamSpec((self.H, d)), "i.b": ParamSpec((self.H,), init="zeros"),
+            "f": ParamSpec((self.H, d)), "f.b": ParamSpec((self.H,), init="ones"),
+            "norm": ParamSpec((v,), init="ones"), "o": ParamSpec((d, v)),
+        }
+
+    def check_sizes(self, dtype: torch.dtype) -> None:
+        if self.dk > 256:
+            raise ValueError(f"matrix_memory: keys of {self.dk} channels; the kernel takes up to 256 (values: any number)")
+
+    def cache_need(self):
+        return StateNeed(shape=(ops.matrix_memory_state_size(self.H, self.dk, self.dv),), dtype="float32")
+
+    def bind(self, tensors: Dict[str, torch.Tensor]) -> None:
+        # one projection [q | k | v | output gate | input gate | forget gate]: a single product per step
+        self.w_all = torch.cat([tensors[n] for n in ("q", "k", "v", "g", "i", "f")], dim=0).contiguous()
+        self.w_o = tensors["o"].contiguous()
+        self.i_b = tensors["i.b"].float().contiguous()
+        self.f_b = tensors["f.b"].float().contiguous()
+        self.norm_w = tensors["norm"].float().contiguous()
+
+    def linear_weights(self):
+        return [self.w_all, (self.w_o, "sum")]
+
+    def forward(self, x, ctx, cache):
+        qk, v = self.H * self.dk, self.H * self.dv
+        proj = ops.linear(ops.resolved(x), self.w_all)
+        y = ops.matrix_memory(proj, 0, qk, 2 * qk, 2 * qk + 2 * v, 2 * qk + 2 * v + self.H, 2 * qk + v, self.i_b, self.f_b,
+                              self.gate_cap, self.norm_w, self.norm_eps, cache.tensor, 0, ctx.qo_indptr, ctx.slot_ids,
+                              self.H, self.dk, self.dv)
         return ops.linear_to_sum(y, self.w_o)

@@ -63,6 +63,22 @@ def safetensors_files(folder) -> List[Path]:
     return files
 
 
+def tensor_shapes(folder) -> Dict[str, Tuple[int, ...]]:
+    """Name -> shape of every tensor in a model folder's safetensors, from the files' headers alone (eight bytes of
+    length, then that many bytes of JSON); no tensor is read."""
+    import struct
+
+    shapes: Dict[str, Tuple[int, ...]] = {}
+    for path in safetensors_files(folder):
+        with open(path, "rb") as f:
+            (length,) = struct.unpack("<Q", f.read(8))
+            header = json.loads(f.read(length))
+        for name, entry in header.items():
+            if name != "__metadata__":
+                shapes[name] = tuple(entry["shape"])
+    return shapes
+
+
 def _final_dtype(spec: ParamSpec, stored: torch.dtype, compute: torch.dtype) -> torch.dtype:
     if spec.kind == "int":
         return torch.int32

@@ -181,3 +181,46 @@ def vobolorn_name_rules(cfg) -> List[NameRule]:
         names = latent if layer.type == "latent_attention" else grouped
         rules += [NameRule(p + ext, p + own) for ext, own in names.items()]
     return rules
+
+
+def kepevik_name_rules(cfg) -> List[NameRule]:
+    """Kepevik checkpoints name a layer's tensors ``l<i>.norm1``, ``norm1b``, ``norm2``, ``norm2b`` (the norms before
+    and behind the two branches), ``l<i>.ls1`` and ``ls2`` (the layer scales, which belong to the norms behind the
+    branches here), ``l<i>.mix.<tensor>`` (a parallel layer: ``l<i>.mix.left.<tensor>`` and ``mix.right.<tensor>``) and
+    ``l<i>.mlp.<tensor>`` (a mixture: ``mlp.e<j>.{gate,up,down}``, ``mlp.router``, ``mlp.correction``,
+    ``mlp.shared.{gate,up,down,sg}``); a bias is the tensor's name with ``.b``.  The output head is the embedding."""
+    L = "l{}."
+    rules = [
+        NameRule("embed", "embed.weight"),
+        NameRule("final.norm", "final_norm.weight"),
+        NameRule(L + "norm1", L + "norm1.weight"),
+        NameRule(L + "norm1b", L + "norm1b.weight"),
+        NameRule(L + "ls1", L + "norm1b.scale"),
+        NameRule(L + "norm2", L + "norm2.weight"),
+        NameRule(L + "norm2b", L + "norm2b.weight"),
+        NameRule(L + "ls2", L + "norm2b.scale"),
+        NameRule(L + "mlp.up", L + "mlp.up.weight"),
+        NameRule(L + "mlp.up.b", L + "mlp.up.bias"),
+        NameRule(L + "mlp.down", L + "mlp.down.weight"),
+        NameRule(L + "mlp.down.b", L + "mlp.down.bias"),
+        NameRule(L + "mlp.router", L + "mlp.router.weight"),
+        NameRule(L + "mlp.correction", L + "mlp.correction"),
+        NameRule(L + "mlp.e{}.gate", L + "mlp.experts.{}.w1.weight"),
+        NameRule(L + "mlp.e{}.up", L + "mlp.experts.{}.w3.weight"),
+        NameRule(L + "mlp.e{}.down", L + "mlp.experts.{}.w2.weight"),
+        NameRule(L + "mlp.shared.gate", L + "mlp.shared.w1.weight"),
+        NameRule(L + "mlp.shared.up", L + "mlp.shared.w3.weight"),
+        NameRule(L + "mlp.shared.down", L + "mlp.shared.w2.weight"),
+        NameRule(L + "mlp.shared.sg", L + "mlp.shared.gate.weight"),
+    ]
+    memory = ["q", "k", "v", "g", "o", "norm", "i", "i.b", "f", "f.b"]
+    left = {"q": "wq.weight", "k": "wk.weight", "o": "wo.weight"}
+    right = ["q", "q.conv", "k", "k.conv", "v", "v.conv", "b", "A_log", "norm", "a1", "a2", "dt_bias", "g1", "g2", "o"]
+    for i, layer in enumerate(cfg.layers):
+        p = f"l{i}.mix."
+        if layer.type == "mlstm":
+            rules += [NameRule(p + n, p + n) for n in memory]
+        else:
+            rules += [NameRule(p + "left." + ext, f"l{i}.left." + own) for ext, own in left.items()]
+            rules += [NameRule(p + "right." + n, f"l{i}.right." + n) for n in right]
+    return rules
