@@ -2,7 +2,7 @@
 bfloat16 weights, synthetic token ids.
 
     python bench.py [--gpus 1] [--steps K] [--warmup W] [--batch 8] [--context 8192] [--layers L]
-                    [--shape 8b|1b|70b] [--workload decode|serve|peaks|small-kernels|attention|products|taluvik|vobolorn]
+                    [--shape 8b|1b|70b] [--workload decode|serve|peaks|small-kernels|attention|products|taluvik|vobolorn|kepevik]
 
 Everything runs through the generation loop: the scheduler admits the requests, cuts their prompts
 into portions under its token budget, and plans every decode step; the step function runs it; the
@@ -28,6 +28,8 @@ a read of 4 GiB with 16-byte loads, a device copy, a loop of MFMA instructions o
 library's large matrix product.  ``--workload small-kernels`` times what a norm kernel adds to a
 replayed graph of large products, without a profiler (under rocprofv3 no dispatch is shorter than
 about 4.6 us, an empty kernel included, so a kernel trace overstates the small kernels of a step).
+``--workload kepevik``: prefill and decode of a Kepevik model (matrix memory, attention beside a delta rule with a
+decay per key channel, routed feed-forwards) beside a Taluvik model of the same layer sizes.
 ``--workload taluvik``: prefill and decode of a Taluvik model (chunked attention with sinks, gated delta
 rule, selective scan) beside a Llama model of the same layer sizes.  ``--workload vobolorn``: the same for a Vobolorn model (grouped-query layers with normed heads, a query factor, mixed
 values and gates, and attention through a latent, over a 32-bit stream).  ``--workload attention``: the decode attention and the merge of its splits alone, by batch size, context and
@@ -84,8 +86,8 @@ def parse_args(argv=None):
     p.add_argument("--points", default="1,64", help="further decode batch sizes, comma separated ('' for none)")
     p.add_argument("--page-size", type=int, default=16)
     p.add_argument("--shape", default="8b", choices=sorted(SHAPES), help="layer sizes (default: the headline's)")
-    p.add_argument("--workload", default="decode", choices=["decode", "serve", "peaks", "small-kernels", "attention", "products", "taluvik", "vobolorn"])
-    p.add_argument("--only", default=None, choices=["taluvik", "vobolorn", "llama"], help="taluvik, vobolorn: measure one of the two models only")
+    p.add_argument("--workload", default="decode", choices=["decode", "serve", "peaks", "small-kernels", "attention", "products", "taluvik", "vobolorn", "kepevik"])
+    p.add_argument("--only", default=None, choices=["taluvik", "vobolorn", "kepevik", "llama"], help="taluvik, vobolorn, kepevik: measure one of the two models only")
     p.add_argument("--token-budget", type=int, default=8192, help="tokens a step may hold (the scheduler cuts prompts to it)")
     p.add_argument("--no-reference-workload", action="store_true",
                    help="leave out the reference's benchmark (2,048-token prompts, 256 new tokens at batch 1, 8, 64)")
@@ -338,6 +340,24 @@ def vobolorn_config(shape: dict, n_layers: int) -> dict:
             "layers": [{"type": turn[i % 4], "mixer": mixers[turn[i % 4]], "mlp": ff} for i in range(n_layers)]}
 
 
+def kepevik_config(shape: dict, n_layers: int) -> dict:
+    """A Kepevik configuration with the layer sizes of ``shape`` (a Llama configuration): the same width, heads and
+    head size.  Matrix-memory layers and parallel layers take turns; the parallel layers' delta rule has half as many
+    key heads as heads, a convolution over four taps and 64 numbers between the two matrices of its decay and of its
+    gate; the first layer's feed-forward is dense with the shape's width inside, the others are mixtures of eight
+    experts of a quarter of that width, of which a token uses two among the eight and one expert that hands its input
+    through, beside a shared expert of a quarter of that width."""
+    D, H, G, dh, ff = shape["hidden_size"], shape["num_attention_heads"], shape["num_key_value_heads"], shape["head_dim"], shape["intermediate_size"]
+    memory = {"heads": H, "dim": dh, "vdim": dh, "gate_cap": 15.0}
+    pair = {"left": {"heads": H, "kv_heads": G, "dim": dh, "vdim": dh, "scale": dh ** -0.5, "rot": {"dims": dh // 2, "base": shape["rope_theta"]}},
+            "right": {"heads": H, "kv_heads": max(H // 2, 1), "dim": dh, "vdim": dh, "conv": 4, "decay_rank": 64, "gate_rank": 64},
+            "left_scale": 0.6, "right_scale": 0.5}
+    moe = {"kind": "moe", "expert": {"ff": ff // 4}, "router": {"experts": 8, "top": 2, "identity": 1}, "shared": {"ff": ff // 4}}
+    return {"architecture": "Kepevik", "vocab": shape["vocab_size"], "width": D, "embedding": {"scale": 1.0}, "norm": {"eps": 1e-6},
+            "layers": [{"type": "mlstm" if i % 2 == 0 else "parallel", "mixer": memory if i % 2 == 0 else pair,
+                        "mlp": {"kind": "dense", "ff": ff} if i == 0 else moe} for i in range(n_layers)]}
+
+
 def taluvik_run(args, shape) -> int:
     """Prefill and decode of a Taluvik (or, ``--workload vobolorn``, a Vobolorn) model beside a Llama model of the
     same layer sizes and number of layers, both with random weights, both through the same engine, scheduler and
@@ -353,12 +373,21 @@ def taluvik_run(args, shape) -> int:
     n_layers = args.layers or 8
     batches = [args.batch] + [int(b) for b in args.points.split(",") if b]
     pages_per_req = -(-max(args.context, args.prefill_tokens) // args.page_size) + 1
-    design = "Vobolorn" if args.workload == "vobolorn" else "Taluvik"
-    configs = {
-        args.workload: (VobolornConfig.from_dict(vobolorn_config(shape, n_layers)) if args.workload == "vobolorn"
-                        else TaluvikConfig.from_dict(taluvik_config(shape, n_layers, chunk=8192))),
-        "llama": LlamaConfig.from_dict(dict(shape, num_hidden_layers=n_layers)),
-    }
+    design = {"vobolorn": "Vobolorn", "kepevik": "Kepevik"}.get(args.workload, "Taluvik")
+    beside = "Llama"
+    if args.workload == "kepevik":
+        # beside the design nearest to it: Taluvik, whose layers hold a delta rule, attention and a recurrence too
+        from torchllms_amd.config.kepevik import KepevikConfig
+
+        beside = "Taluvik"
+        configs = {"kepevik": KepevikConfig.from_dict(kepevik_config(shape, n_layers)),
+                   "taluvik": TaluvikConfig.from_dict(taluvik_config(shape, n_layers, chunk=8192))}
+    else:
+        configs = {
+            args.workload: (VobolornConfig.from_dict(vobolorn_config(shape, n_layers)) if args.workload == "vobolorn"
+                            else TaluvikConfig.from_dict(taluvik_config(shape, n_layers, chunk=8192))),
+            "llama": LlamaConfig.from_dict(dict(shape, num_hidden_layers=n_layers)),
+        }
     if args.only:
         configs = {k: v for k, v in configs.items() if k == args.only}
     new_tokens = 1 + 2 + 3 + args.warmup + args.steps + 1
@@ -381,11 +410,11 @@ def taluvik_run(args, shape) -> int:
     first = next(iter(out.values()))
     ms = first[f"decode_b{args.batch}"]["ms_per_step"]
     print(json.dumps({
-        "metric": f"decode tok/s, batch {args.batch}, context {args.context}, {design} beside Llama at {SHAPE_NAMES[args.shape]} layer sizes, {n_layers} layers",
+        "metric": f"decode tok/s, batch {args.batch}, context {args.context}, {design} beside {beside} at {SHAPE_NAMES[args.shape]} layer sizes, {n_layers} layers",
         "value": first[f"decode_b{args.batch}"]["tokens_per_s"], "unit": "tokens/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
         "ms_per_step": ms, "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
         "dtype": "bf16" if args.dtype == "bfloat16" else "fp32", "data": "synthetic: random-init weights, random token ids",
-        "config": {"model": f"{design} and Llama at {SHAPE_NAMES[args.shape]} layer sizes", "global_batch": args.batch, "seq_len": args.context,
+        "config": {"model": f"{design} and {beside} at {SHAPE_NAMES[args.shape]} layer sizes", "global_batch": args.batch, "seq_len": args.context,
                    "parallelism": "single GPU", "n_layers": n_layers, "page_size": args.page_size},
         "models": out,
     }))
@@ -621,7 +650,7 @@ def main(argv=None) -> int:
         return products_run(args, shape)
     if args.workload == "peaks":
         return peaks_run(args)
-    if args.workload in ("taluvik", "vobolorn"):
+    if args.workload in ("taluvik", "vobolorn", "kepevik"):
         return taluvik_run(args, shape)
     import torch
 

@@ -66,86 +66,273 @@ router_topk_kernel(const float* __restrict__ z, int z_stride, const float* __res
   }
 }
 
-// ----------------------------------------------------------------------------- experts, a (token, choice) at a time
-// mid[p, f] = T(silu(Wg[e] x) * (Wu[e] x)) for the pair p = (token t, choice j), e = ids[p] < n_experts; pairs whose
-// expert hands its input through are left alone.  w_gu [E][2F][D] (an expert's gate rows, then its up rows).  A wave
-// takes an output at a time, its lanes the row's elements V at a time; the sums have an order fixed by D alone.
-constexpr int kPairThreads = 256;
+// ----------------------------------------------------------------------------- experts over their gathered rows
+// The (token, choice) pairs lie in the order of their experts (expert_gather below): rows[offsets[e] .. offsets[e + 1]]
+// are the inputs of expert e.  A block takes some outputs of one expert and walks that expert's rows R at a time: the
+// rows go to LDS, a wave takes an output at a time, reads its weights once (V elements a lane) and multiplies them
+// with all R rows, so an expert's weights are read once per R rows however many tokens chose it.  Every row's sum has
+// an order fixed by the row's width alone, whatever lies beside it.
+constexpr int kRowsThreads = 256;
+constexpr int kRowsAtOnce = 8;
+
+// mid[r, f] = T(silu(Wg[e][f] . x_r) * (Wu[e][f] . x_r)); w_gu [E][2F][D] (an expert's gate rows, then its up rows).
 template <typename T, int V>
-__global__ void __launch_bounds__(kPairThreads)
-expert_glu_pairs_kernel(const T* __restrict__ x, const T* __restrict__ w_gu, const int32_t* __restrict__ ids, int top, int n_experts,
-                        T* __restrict__ mid, int D, int F, int f_per_block) {
-  extern __shared__ __attribute__((aligned(16))) float x_l[];
-  const int p = blockIdx.x;
-  const int e = ids[p];
-  if (e >= n_experts) return;
-  const T* xr = x + (size_t)(p / top) * D;
-  for (int d = threadIdx.x; d < D; d += kPairThreads) x_l[d] = to_f32(xr[d]);
-  __syncthreads();
+__global__ void __launch_bounds__(kRowsThreads)
+expert_glu_rows_kernel(const T* __restrict__ rows, const T* __restrict__ w_gu, const int32_t* __restrict__ offsets,
+                       T* __restrict__ mid, int D, int F, int f_per_block, int at_once) {
+  extern __shared__ __attribute__((aligned(16))) unsigned char lds_raw[];
+  T* x_l = reinterpret_cast<T*>(lds_raw);  // [at_once][D]
+  const int e = blockIdx.x;
+  const int lo = offsets[e], hi = offsets[e + 1];
+  if (lo == hi) return;
   const int wave = threadIdx.x / kWave, lane = threadIdx.x % kWave;
-  const int f_end = min(F, (blockIdx.y + 1) * f_per_block);
+  const int f_begin = blockIdx.y * f_per_block, f_end = min(F, f_begin + f_per_block);
   const T* wg = w_gu + (size_t)e * 2 * F * D;
-  for (int f = blockIdx.y * f_per_block + wave; f < f_end; f += kPairThreads / kWave) {
-    const T* g_row = wg + (size_t)f * D;
-    const T* u_row = wg + (size_t)(F + f) * D;
-    float ag = 0.f, au = 0.f;
-    for (int d0 = lane * V; d0 < D; d0 += kWave * V) {
-      struct alignas(sizeof(T) * V) Vec { T e[V]; };
-      const Vec gv = *reinterpret_cast<const Vec*>(g_row + d0);
-      const Vec uv = *reinterpret_cast<const Vec*>(u_row + d0);
+  struct alignas(sizeof(T) * V) Vec { T e[V]; };
+  for (int r0 = lo; r0 < hi; r0 += at_once) {
+    const int nr = min(at_once, hi - r0);
+    __syncthreads();
+    for (int i = threadIdx.x * V; i < nr * D; i += kRowsThreads * V)
+      *reinterpret_cast<Vec*>(x_l + i) = *reinterpret_cast<const Vec*>(rows + (size_t)r0 * D + i);
+    __syncthreads();
+    for (int f = f_begin + wave; f < f_end; f += kRowsThreads / kWave) {
+      const T* g_row = wg + (size_t)f * D;
+      const T* u_row = wg + (size_t)(F + f) * D;
+      float ag[kRowsAtOnce], au[kRowsAtOnce];
 #pragma unroll
-      for (int i = 0; i < V; ++i) {
-        ag = fmaf(to_f32(gv.e[i]), x_l[d0 + i], ag);
-        au = fmaf(to_f32(uv.e[i]), x_l[d0 + i], au);
+      for (int r = 0; r < kRowsAtOnce; ++r) ag[r] = au[r] = 0.f;
+#pragma unroll 4
+      for (int d0 = lane * V; d0 < D; d0 += kWave * V) {  // (unrolled: the loads of four rounds are asked for together)
+        const Vec gv = *reinterpret_cast<const Vec*>(g_row + d0);
+        const Vec uv = *reinterpret_cast<const Vec*>(u_row + d0);
+        float gf[V], uf[V];
+#pragma unroll
+        for (int i = 0; i < V; ++i) { gf[i] = to_f32(gv.e[i]); uf[i] = to_f32(uv.e[i]); }
+#pragma unroll
+        for (int r = 0; r < kRowsAtOnce; ++r) {
+          if (r < nr) {
+            const Vec xv = *reinterpret_cast<const Vec*>(x_l + r * D + d0);
+#pragma unroll
+            for (int i = 0; i < V; ++i) {
+              const float xe = to_f32(xv.e[i]);
+              ag[r] = fmaf(gf[i], xe, ag[r]);
+              au[r] = fmaf(uf[i], xe, au[r]);
+            }
+          }
+        }
+      }
+#pragma unroll
+      for (int r = 0; r < kRowsAtOnce; ++r) {
+        if (r < nr) {
+          const float g = wave_sum(ag[r]), u = wave_sum(au[r]);
+          if (lane == 0) mid[(size_t)(r0 + r) * F + f] = from_f32<T>(silu_r(g) * u);
+        }
       }
     }
-    ag = wave_sum(ag);
-    au = wave_sum(au);
-    if (lane == 0) mid[(size_t)p * F + f] = from_f32<T>(silu_r(ag) * au);
   }
 }
 
-// out[t, d] = T(sum_j w[t, j] * (e_j < n_experts ? Wd[e_j][d] . mid[t, j] : x[t, d]) + sigmoid(sg[t]) * shared[t, d]);
-// w_d [E][D][F]; shared (or null) [n, D] with its gate's 32-bit pre-activation sg[t * sg_stride].  The pairs of a token
-// are added in the order of its choices.
+// y[r, d] = Wd[e][d] . mid_r in 32-bit; w_d [E][D][F].
 template <typename T, int V>
-__global__ void __launch_bounds__(kPairThreads)
-expert_down_pairs_kernel(const T* __restrict__ mid, const T* __restrict__ w_d, const int32_t* __restrict__ ids,
-                         const float* __restrict__ weights, int top, int n_experts, const T* __restrict__ x,
-                         const T* __restrict__ shared, const float* __restrict__ sg, int sg_stride, T* __restrict__ out, int D,
-                         int F, int d_per_block) {
-  extern __shared__ __attribute__((aligned(16))) float mid_l[];  // [top][F]
-  const int t = blockIdx.x;
-  for (int i = threadIdx.x; i < top * F; i += kPairThreads) {
-    const int j = i / F;
-    mid_l[i] = ids[(size_t)t * top + j] < n_experts ? to_f32(mid[(size_t)t * top * F + i]) : 0.f;
+__global__ void __launch_bounds__(kRowsThreads)
+expert_down_rows_kernel(const T* __restrict__ mid, const T* __restrict__ w_d, const int32_t* __restrict__ offsets,
+                        float* __restrict__ y, int D, int F, int d_per_block, int at_once) {
+  extern __shared__ __attribute__((aligned(16))) unsigned char lds_raw[];
+  T* m_l = reinterpret_cast<T*>(lds_raw);  // [at_once][F]
+  const int e = blockIdx.x;
+  const int lo = offsets[e], hi = offsets[e + 1];
+  if (lo == hi) return;
+  const int wave = threadIdx.x / kWave, lane = threadIdx.x % kWave;
+  const int d_begin = blockIdx.y * d_per_block, d_end = min(D, d_begin + d_per_block);
+  struct alignas(sizeof(T) * V) Vec { T e[V]; };
+  for (int r0 = lo; r0 < hi; r0 += at_once) {
+    const int nr = min(at_once, hi - r0);
+    __syncthreads();
+    for (int i = threadIdx.x * V; i < nr * F; i += kRowsThreads * V)
+      *reinterpret_cast<Vec*>(m_l + i) = *reinterpret_cast<const Vec*>(mid + (size_t)r0 * F + i);
+    __syncthreads();
+    for (int d = d_begin + wave; d < d_end; d += kRowsThreads / kWave) {
+      const T* row = w_d + ((size_t)e * D + d) * F;
+      float acc[kRowsAtOnce];
+#pragma unroll
+      for (int r = 0; r < kRowsAtOnce; ++r) acc[r] = 0.f;
+#pragma unroll 4
+      for (int f0 = lane * V; f0 < F; f0 += kWave * V) {
+        const Vec wv = *reinterpret_cast<const Vec*>(row + f0);
+        float wf[V];
+#pragma unroll
+        for (int i = 0; i < V; ++i) wf[i] = to_f32(wv.e[i]);
+#pragma unroll
+        for (int r = 0; r < kRowsAtOnce; ++r) {
+          if (r < nr) {
+            const Vec mv = *reinterpret_cast<const Vec*>(m_l + r * F + f0);
+#pragma unroll
+            for (int i = 0; i < V; ++i) acc[r] = fmaf(wf[i], to_f32(mv.e[i]), acc[r]);
+          }
+        }
+      }
+#pragma unroll
+      for (int r = 0; r < kRowsAtOnce; ++r) {
+        if (r < nr) {
+          const float v = wave_sum(acc[r]);
+          if (lane == 0) y[(size_t)(r0 + r) * D + d] = v;
+        }
+      }
+    }
+  }
+}
+
+// The same two products for bfloat16 rows of up to NI * 512 elements, with the weights held in registers: a wave takes
+// one output, asks for its whole weight row (gate and up row) at once, 16 bytes a lane and round, and then walks the
+// expert's rows, at_once of them in LDS at a time.  The weights are read once however many rows the expert has, and every
+// load of a wave is in flight together.  GLU: w [E][2N][K], mid[r, n] = silu(gate) * up; else w [E][N][K], y[r, n] in 32-bit.
+// Each row's sum is taken in the order of the kernels above (a lane its rounds in ascending order, then the lanes).
+typedef __bf16 bf16x8_r __attribute__((ext_vector_type(8)));
+constexpr int kHeldRows = 4;
+template <int NI, bool GLU>
+__global__ void __launch_bounds__(kRowsThreads)
+expert_rows_held_kernel(const bf16_t* __restrict__ rows, const bf16_t* __restrict__ w, const int32_t* __restrict__ offsets,
+                        bf16_t* __restrict__ mid, float* __restrict__ y, int K, int N, int at_once) {
+  extern __shared__ __attribute__((aligned(16))) unsigned char lds_raw[];
+  bf16_t* x_l = reinterpret_cast<bf16_t*>(lds_raw);  // [at_once][K]
+  const int e = blockIdx.x;
+  const int lo = offsets[e], hi = offsets[e + 1];
+  if (lo == hi) return;
+  const int wave = threadIdx.x / kWave, lane = threadIdx.x % kWave;
+  const int n = blockIdx.y * (kRowsThreads / kWave) + wave;
+  const bool live = n < N;
+  const bf16_t* g_row = w + ((size_t)e * (GLU ? 2 : 1) * N + (live ? n : 0)) * K;
+  const bf16_t* u_row = g_row + (size_t)N * K;
+  bf16x8_r gw[NI], uw[GLU ? NI : 1];
+#pragma unroll
+  for (int it = 0; it < NI; ++it) {
+    const int d0 = (it * kWave + lane) * 8;
+    const int at = d0 < K ? d0 : 0;
+    gw[it] = *reinterpret_cast<const bf16x8_r*>(g_row + at);
+    if (GLU) uw[it] = *reinterpret_cast<const bf16x8_r*>(u_row + at);
+  }
+  for (int r0 = lo; r0 < hi; r0 += at_once) {
+    const int nr = min(at_once, hi - r0);
+    __syncthreads();
+    for (int i = threadIdx.x * 8; i < nr * K; i += kRowsThreads * 8)
+      *reinterpret_cast<bf16x8_r*>(x_l + i) = *reinterpret_cast<const bf16x8_r*>(rows + (size_t)r0 * K + i);
+    __syncthreads();
+    float ag[kHeldRows], au[kHeldRows];
+#pragma unroll
+    for (int r = 0; r < kHeldRows; ++r) ag[r] = au[r] = 0.f;
+#pragma unroll
+    for (int it = 0; it < NI; ++it) {
+      const int d0 = (it * kWave + lane) * 8;
+      if (d0 < K) {
+#pragma unroll
+        for (int r = 0; r < kHeldRows; ++r) {
+          if (r < nr) {
+            const bf16x8_r xv = *reinterpret_cast<const bf16x8_r*>(x_l + r * K + d0);
+#pragma unroll
+            for (int i = 0; i < 8; ++i) {
+              const float xe = (float)xv[i];
+              ag[r] = fmaf((float)gw[it][i], xe, ag[r]);
+              if (GLU) au[r] = fmaf((float)uw[it][i], xe, au[r]);
+            }
+          }
+        }
+      }
+    }
+#pragma unroll
+    for (int r = 0; r < kHeldRows; ++r) {
+      if (r < nr) {
+        const float g = wave_sum(ag[r]);
+        if (GLU) {
+          const float u = wave_sum(au[r]);
+          if (live && lane == 0) mid[(size_t)(r0 + r) * N + n] = from_f32<bf16_t>(silu_r(g) * u);
+        } else {
+          if (live && lane == 0) y[(size_t)(r0 + r) * N + n] = g;
+        }
+      }
+    }
+  }
+}
+
+template <bool GLU>
+static int launch_rows_held(const void* rows, const void* w, const int32_t* offsets, int n_experts, void* mid, float* y, int K, int N,
+                            int max_rows, hipStream_t stream) {
+  int at_once = 1;
+  while (at_once < kHeldRows && at_once < max_rows) at_once *= 2;
+  while (at_once > 1 && (size_t)at_once * K * 2 > 32 * 1024) at_once /= 2;
+  const size_t lds = (size_t)at_once * K * 2;
+  const dim3 grid(n_experts, (N + kRowsThreads / kWave - 1) / (kRowsThreads / kWave));
+  const int rounds = (K + kWave * 8 - 1) / (kWave * 8);
+#define TL_HELD(NI) expert_rows_held_kernel<NI, GLU><<<grid, kRowsThreads, lds, stream>>>((const bf16_t*)rows, (const bf16_t*)w, offsets, (bf16_t*)mid, y, K, N, at_once)
+  if (rounds <= 1) TL_HELD(1);
+  else if (rounds <= 2) TL_HELD(2);
+  else if (rounds <= 4) TL_HELD(4);
+  else if (rounds <= 8) TL_HELD(8);
+  else TL_HELD(16);
+#undef TL_HELD
+  return tl_check_launch("expert_rows_held");
+}
+// The widest rows the kernel with held weights takes, in elements (bfloat16, a multiple of 8).
+constexpr int kHeldMaxWidth = 16 * kWave * 8;
+
+// ----------------------------------------------------------------------------- experts, the rows of each side by side
+// The (token, choice) pairs are put in the order of their experts, so that an expert's rows lie side by side and its
+// weights are read once for all of them.  counts[e]: how many pairs chose output e.
+__global__ void __launch_bounds__(256)
+expert_count_kernel(const int32_t* __restrict__ ids, int pairs, int32_t* __restrict__ counts) {
+  for (int p = blockIdx.x * blockDim.x + threadIdx.x; p < pairs; p += gridDim.x * blockDim.x) atomicAdd(&counts[ids[p]], 1);
+}
+
+// offsets[e] = counts[0] + .. + counts[e - 1] (and the total at n_out); cursor[e] = 0.  One thread: n_out is small.
+__global__ void expert_offsets_kernel(const int32_t* __restrict__ counts, int n_out, int32_t* __restrict__ offsets,
+                                      int32_t* __restrict__ cursor) {
+  if (threadIdx.x != 0 || blockIdx.x != 0) return;
+  int total = 0;
+  for (int e = 0; e < n_out; ++e) {
+    offsets[e] = total;
+    cursor[e] = 0;
+    total += counts[e];
+  }
+  offsets[n_out] = total;
+}
+
+// A block a pair: the pair takes the next free row of its expert's range (which of an expert's pairs gets which row
+// depends on timing; a row's result does not depend on where it lies), remembers it in pos[p], and its token's row of
+// x is copied there.
+template <typename T>
+__global__ void __launch_bounds__(256)
+expert_gather_kernel(const T* __restrict__ x, const int32_t* __restrict__ ids, const int32_t* __restrict__ offsets,
+                     int32_t* __restrict__ cursor, int top, int32_t* __restrict__ pos, T* __restrict__ rows, int D) {
+  __shared__ int at_l;
+  const int p = blockIdx.x;
+  if (threadIdx.x == 0) {
+    const int e = ids[p];
+    at_l = offsets[e] + atomicAdd(&cursor[e], 1);
+    pos[p] = at_l;
   }
   __syncthreads();
-  const int wave = threadIdx.x / kWave, lane = threadIdx.x % kWave;
-  const int d_end = min(D, (blockIdx.y + 1) * d_per_block);
+  const T* src = x + (size_t)(p / top) * D;
+  T* dst = rows + (size_t)at_l * D;
+  for (int d = threadIdx.x; d < D; d += blockDim.x) dst[d] = src[d];
+}
+
+// out[t, d] = T(sum_j w[t, j] * (e_j < n_experts ? y[pos[t, j], d] : x[t, d]) + sigmoid(sg[t]) * shared[t, d]): the
+// experts' results (32-bit, or of the tensors' dtype) back in the order of the tokens, weighted and added in the order of a token's choices.
+template <typename T, typename YT>
+__global__ void __launch_bounds__(256)
+expert_combine_kernel(const YT* __restrict__ y, const int32_t* __restrict__ pos, const int32_t* __restrict__ ids,
+                      const float* __restrict__ weights, int top, int n_experts, const T* __restrict__ x,
+                      const T* __restrict__ shared, const float* __restrict__ sg, int sg_stride, T* __restrict__ out, int D) {
+  const int t = blockIdx.x;
   const float share = shared ? sigmoid_r(sg[(size_t)t * sg_stride]) : 0.f;
-  for (int d = blockIdx.y * d_per_block + wave; d < d_end; d += kPairThreads / kWave) {
+  for (int d = threadIdx.x; d < D; d += blockDim.x) {
     float total = 0.f;
     for (int j = 0; j < top; ++j) {
       const int e = ids[(size_t)t * top + j];
       const float wj = weights[(size_t)t * top + j];
-      if (e >= n_experts) {
-        total += wj * to_f32(x[(size_t)t * D + d]);
-        continue;
-      }
-      const T* row = w_d + ((size_t)e * D + d) * F;
-      const float* m = mid_l + j * F;
-      float acc = 0.f;
-      for (int f0 = lane * V; f0 < F; f0 += kWave * V) {
-        struct alignas(sizeof(T) * V) Vec { T e[V]; };
-        const Vec wv = *reinterpret_cast<const Vec*>(row + f0);
-#pragma unroll
-        for (int i = 0; i < V; ++i) acc = fmaf(to_f32(wv.e[i]), m[f0 + i], acc);
-      }
-      total += wj * wave_sum(acc);
+      total += wj * (e < n_experts ? to_f32(y[(size_t)pos[(size_t)t * top + j] * D + d]) : to_f32(x[(size_t)t * D + d]));
     }
     if (shared) total += share * to_f32(shared[(size_t)t * D + d]);
-    if (lane == 0) out[(size_t)t * D + d] = from_f32<T>(total);
+    out[(size_t)t * D + d] = from_f32<T>(total);
   }
 }
 
@@ -218,61 +405,110 @@ TL_EXPORT int tl_router_topk(const float* z, int z_stride, const float* correcti
   return tl_check_launch("router_topk");
 }
 
-TL_EXPORT int tl_expert_glu_pairs(const void* x, const void* w_gu, const int32_t* ids, int top, int n_experts, void* mid, int n,
-                                  int D, int F, int dtype, hipStream_t stream) {
-  TL_REQUIRE(n >= 0 && top > 0 && n_experts >= 0 && D > 0 && F > 0, "expert_glu_pairs: bad sizes");
-  TL_REQUIRE((long long)n * top <= 0x7fffffff, "expert_glu_pairs: too many pairs a step");
-  if (n == 0 || n_experts == 0) return TL_OK;
-  const size_t lds = (size_t)D * sizeof(float);
+// How many of an expert's rows a block holds in LDS at once: no more than any expert can have (`max_rows`, the step's
+// pairs), and no more than 32 KB of them, so that several blocks share a CU and hide each other's trips to memory (an
+// expert with more rows is walked in several passes; a block's few weight rows come from the caches then).
+static int rows_at_once(int width, int elem, int max_rows) {
+  int r = 1;
+  while (r < kRowsAtOnce && r < max_rows) r *= 2;
+  while (r > 1 && (size_t)r * width * elem > 32 * 1024) r /= 2;
+  return r;
+}
+// Outputs a block takes: as few as leave eight blocks a CU among the experts that can be in use.
+static int outputs_per_block(int n_experts, int n_out, int max_rows) {
+  const int active = max_rows < n_experts ? (max_rows > 0 ? max_rows : 1) : n_experts;
+  const int want_blocks = 8 * tl_device_facts().compute_units;
+  int per = (int)(((long long)n_out * active + want_blocks - 1) / want_blocks);
+  const int waves = kRowsThreads / kWave;
+  per = (per + waves - 1) / waves * waves;
+  return per < waves ? waves : per;
+}
+
+// rows [pairs, D] in the order of their experts, offsets [n_experts + 1 ..]; mid [pairs, F].
+TL_EXPORT int tl_expert_glu_rows(const void* rows, const void* w_gu, const int32_t* offsets, int n_experts, void* mid, int D, int F,
+                                 int max_rows, int dtype, hipStream_t stream) {
+  TL_REQUIRE(n_experts >= 0 && D > 0 && F > 0 && max_rows >= 0, "expert_glu_rows: bad sizes");
+  if (n_experts == 0 || max_rows == 0) return TL_OK;
+  if (dtype != TL_F32 && dtype != TL_BF16) return tl_fail(TL_ERR_ARG, "expert_glu_rows: unknown dtype %d", dtype);
+  if (dtype == TL_BF16 && D % 8 == 0 && D <= kHeldMaxWidth)
+    return launch_rows_held<true>(rows, w_gu, offsets, n_experts, mid, nullptr, D, F, max_rows, stream);
+  const int elem = dtype == TL_F32 ? 4 : 2;
+  const int at_once = rows_at_once(D, elem, max_rows);
+  const size_t lds = (size_t)at_once * D * elem;
   if (lds > (size_t)tl_device_facts().lds_bytes)
-    return tl_fail(TL_ERR_UNSUPPORTED, "expert_glu_pairs: rows of %d elements do not fit the LDS", D);
-  // blocks: enough to fill the GPU with few pairs, not more outputs a block than that needs
-  const int pairs = n * top;
-  int f_per_block = F;
-  const int want_blocks = 4 * tl_device_facts().compute_units;
-  if (pairs < want_blocks) f_per_block = max(kPairThreads / kWave, (int)(((long long)F * pairs + want_blocks - 1) / want_blocks));
-  const dim3 grid(pairs, (F + f_per_block - 1) / f_per_block);
-#define TL_GLU(T, V) expert_glu_pairs_kernel<T, V><<<grid, kPairThreads, lds, stream>>>((const T*)x, (const T*)w_gu, ids, top, n_experts, (T*)mid, D, F, f_per_block)
+    return tl_fail(TL_ERR_UNSUPPORTED, "expert_glu_rows: rows of %d elements do not fit the LDS", D);
+  const int per = outputs_per_block(n_experts, F, max_rows);
+  const dim3 grid(n_experts, (F + per - 1) / per);
+#define TL_GLU(T, V) expert_glu_rows_kernel<T, V><<<grid, kRowsThreads, lds, stream>>>((const T*)rows, (const T*)w_gu, offsets, (T*)mid, D, F, per, at_once)
   if (dtype == TL_F32) {
     if (D % 4 == 0) TL_GLU(float, 4);
     else TL_GLU(float, 1);
-  } else if (dtype == TL_BF16) {
+  } else {
     if (D % 8 == 0) TL_GLU(bf16_t, 8);
     else TL_GLU(bf16_t, 1);
-  } else {
-    return tl_fail(TL_ERR_ARG, "expert_glu_pairs: unknown dtype %d", dtype);
   }
 #undef TL_GLU
-  return tl_check_launch("expert_glu_pairs");
+  return tl_check_launch("expert_glu_rows");
 }
 
-TL_EXPORT int tl_expert_down_pairs(const void* mid, const void* w_d, const int32_t* ids, const float* weights, int top,
-                                   int n_experts, const void* x, const void* shared, const float* sg, int sg_stride, void* out,
-                                   int n, int D, int F, int dtype, hipStream_t stream) {
-  TL_REQUIRE(n >= 0 && top > 0 && n_experts >= 0 && D > 0 && F > 0, "expert_down_pairs: bad sizes");
-  TL_REQUIRE(shared == nullptr || sg != nullptr, "expert_down_pairs: a shared expert without its gate");
-  if (n == 0) return TL_OK;
-  const size_t lds = (size_t)top * F * sizeof(float);
+// mid [pairs, F] in the order of their experts; y [pairs, D] float.
+TL_EXPORT int tl_expert_down_rows(const void* mid, const void* w_d, const int32_t* offsets, int n_experts, float* y, int D, int F,
+                                  int max_rows, int dtype, hipStream_t stream) {
+  TL_REQUIRE(n_experts >= 0 && D > 0 && F > 0 && max_rows >= 0, "expert_down_rows: bad sizes");
+  if (n_experts == 0 || max_rows == 0) return TL_OK;
+  if (dtype != TL_F32 && dtype != TL_BF16) return tl_fail(TL_ERR_ARG, "expert_down_rows: unknown dtype %d", dtype);
+  if (dtype == TL_BF16 && F % 8 == 0 && F <= kHeldMaxWidth)
+    return launch_rows_held<false>(mid, w_d, offsets, n_experts, nullptr, y, F, D, max_rows, stream);
+  const int elem = dtype == TL_F32 ? 4 : 2;
+  const int at_once = rows_at_once(F, elem, max_rows);
+  const size_t lds = (size_t)at_once * F * elem;
   if (lds > (size_t)tl_device_facts().lds_bytes)
-    return tl_fail(TL_ERR_UNSUPPORTED, "expert_down_pairs: %d choices of %d elements do not fit the LDS", top, F);
-  int d_per_block = D;
-  const int want_blocks = 4 * tl_device_facts().compute_units;
-  if (n < want_blocks) d_per_block = max(kPairThreads / kWave, (int)(((long long)D * n + want_blocks - 1) / want_blocks));
-  const dim3 grid(n, (D + d_per_block - 1) / d_per_block);
-#define TL_DOWN(T, V)                                                                                                        \
-  expert_down_pairs_kernel<T, V><<<grid, kPairThreads, lds, stream>>>((const T*)mid, (const T*)w_d, ids, weights, top, n_experts, \
-                                                                      (const T*)x, (const T*)shared, sg, sg_stride, (T*)out, D, F, d_per_block)
+    return tl_fail(TL_ERR_UNSUPPORTED, "expert_down_rows: rows of %d elements do not fit the LDS", F);
+  const int per = outputs_per_block(n_experts, D, max_rows);
+  const dim3 grid(n_experts, (D + per - 1) / per);
+#define TL_DOWN(T, V) expert_down_rows_kernel<T, V><<<grid, kRowsThreads, lds, stream>>>((const T*)mid, (const T*)w_d, offsets, y, D, F, per, at_once)
   if (dtype == TL_F32) {
     if (F % 4 == 0) TL_DOWN(float, 4);
     else TL_DOWN(float, 1);
-  } else if (dtype == TL_BF16) {
+  } else {
     if (F % 8 == 0) TL_DOWN(bf16_t, 8);
     else TL_DOWN(bf16_t, 1);
-  } else {
-    return tl_fail(TL_ERR_ARG, "expert_down_pairs: unknown dtype %d", dtype);
   }
 #undef TL_DOWN
-  return tl_check_launch("expert_down_pairs");
+  return tl_check_launch("expert_down_rows");
+}
+
+// counts, cursor: n_out int32 each (counts zeroed by the caller); offsets: n_out + 1; pos: n * top; rows [n * top, D].
+TL_EXPORT int tl_expert_gather(const void* x, const int32_t* ids, int n, int top, int n_out, int32_t* counts, int32_t* offsets,
+                               int32_t* cursor, int32_t* pos, void* rows, int D, int dtype, hipStream_t stream) {
+  TL_REQUIRE(n >= 0 && top > 0 && n_out > 0 && D > 0, "expert_gather: bad sizes");
+  TL_REQUIRE((long long)n * top <= 0x7fffffff, "expert_gather: too many pairs a step");
+  if (n == 0) return TL_OK;
+  if (dtype != TL_F32 && dtype != TL_BF16) return tl_fail(TL_ERR_ARG, "expert_gather: unknown dtype %d", dtype);
+  const int pairs = n * top;
+  expert_count_kernel<<<(pairs + 255) / 256 < 1024 ? (pairs + 255) / 256 : 1024, 256, 0, stream>>>(ids, pairs, counts);
+  expert_offsets_kernel<<<1, 64, 0, stream>>>(counts, n_out, offsets, cursor);
+  if (dtype == TL_F32) expert_gather_kernel<float><<<pairs, 256, 0, stream>>>((const float*)x, ids, offsets, cursor, top, pos, (float*)rows, D);
+  else expert_gather_kernel<bf16_t><<<pairs, 256, 0, stream>>>((const bf16_t*)x, ids, offsets, cursor, top, pos, (bf16_t*)rows, D);
+  return tl_check_launch("expert_gather");
+}
+
+// y: the experts' results in the order of the gathered rows, 32-bit (y_f32) or of the tensors' dtype.
+TL_EXPORT int tl_expert_combine(const void* y, int y_f32, const int32_t* pos, const int32_t* ids, const float* weights, int top,
+                                int n_experts, const void* x, const void* shared, const float* sg, int sg_stride, void* out, int n,
+                                int D, int dtype, hipStream_t stream) {
+  TL_REQUIRE(n >= 0 && top > 0 && n_experts >= 0 && D > 0, "expert_combine: bad sizes");
+  TL_REQUIRE(shared == nullptr || sg != nullptr, "expert_combine: a shared expert without its gate");
+  if (n == 0) return TL_OK;
+#define TL_COMBINE(T, YT)                                                                                                   \
+  expert_combine_kernel<T, YT><<<n, 256, 0, stream>>>((const YT*)y, pos, ids, weights, top, n_experts, (const T*)x, (const T*)shared, \
+                                                      sg, sg_stride, (T*)out, D)
+  if (dtype == TL_F32) TL_COMBINE(float, float);
+  else if (dtype == TL_BF16 && y_f32) TL_COMBINE(bf16_t, float);
+  else if (dtype == TL_BF16) TL_COMBINE(bf16_t, bf16_t);
+  else return tl_fail(TL_ERR_ARG, "expert_combine: unknown dtype %d", dtype);
+#undef TL_COMBINE
+  return tl_check_launch("expert_combine");
 }
 
 TL_EXPORT int tl_bias_gelu(void* x, const void* bias, int n, int width, int dtype, hipStream_t stream) {

@@ -43,8 +43,10 @@ _CORE_SIGNATURES = {
     "tl_gated_delta": [_P, _I, _P, _I, _I, _I, _I, _P, _P, _P, _F, _P, _I64, _P, _P, _P, _I, _I, _I, _I, _I, _I, _P, _I, _P, _I, _I, _P, _I, _P],
     "tl_matrix_memory": [_P, _I, _I, _I, _I, _I, _I, _P, _P, _F, _P, _I, _I, _P, _F, _P, _I64, _P, _P, _P, _I, _I, _I, _I, _I, _P, _P, _I, _P],
     "tl_router_topk": [_P, _I, _P, _I, _I, _I, _P, _P, _P],
-    "tl_expert_glu_pairs": [_P, _P, _P, _I, _I, _P, _I, _I, _I, _I, _P],
-    "tl_expert_down_pairs": [_P, _P, _P, _P, _I, _I, _P, _P, _P, _I, _P, _I, _I, _I, _I, _P],
+    "tl_expert_glu_rows": [_P, _P, _P, _I, _P, _I, _I, _I, _I, _P],
+    "tl_expert_down_rows": [_P, _P, _P, _I, _P, _I, _I, _I, _I, _P],
+    "tl_expert_gather": [_P, _P, _I, _I, _I, _P, _P, _P, _P, _P, _I, _I, _P],
+    "tl_expert_combine": [_P, _I, _P, _P, _P, _I, _I, _P, _P, _P, _I, _P, _I, _I, _I, _P],
     "tl_bias_gelu": [_P, _P, _I, _I, _I, _P],
     "tl_weighted_pair": [_P, _F, _P, _F, _P, _I64, _I, _P],
     "tl_post_norm_add_norm": [_P, _P, _P, _F, _P, _F, _P, _I, _I, _I, _P],

@@ -13,7 +13,7 @@ a module's own helpers and tables stay in the module.
                      write, short convolutions, selective scan, gated delta rule, matrix memory
 ``head_ops``         branches normed into a 32-bit stream, heads prepared before the scores (weighted norm, partial
                      rotation, query factor, mixed values), gates, packing for attention through a latent, logit cap
-``routed_ops``       router (softmax scores, corrected choice), experts a (token, choice) at a time, bias with the
+``routed_ops``       router (softmax scores, corrected choice), experts over the rows that chose them, bias with the
                      exact gelu, the norm behind a branch together with the norm before the next
 ``sampling_ops``     the sampling kernel
 """
@@ -121,8 +121,10 @@ from .head_ops import (  # noqa: F401
 from .routed_ops import (  # noqa: F401
     ROUTER_MAX_OUTPUTS,
     bias_gelu_,
-    expert_down_pairs,
-    expert_glu_pairs,
+    expert_combine,
+    expert_down_rows,
+    expert_gather,
+    expert_glu_rows,
     post_norm_add_norm,
     router_topk,
     weighted_pair,

@@ -1,5 +1,6 @@
-"""Kernels of a routed feed-forward (router with softmax scores and a correction for the choice, experts a
-(token, choice) at a time, experts that hand their input through, a shared expert with a gate), of a dense
+"""Kernels of a routed feed-forward (router with softmax scores and a correction for the choice, the (token, choice)
+pairs gathered in the order of their experts, experts over their rows, experts that hand their input through, a
+shared expert with a gate), of a dense
 feed-forward with biases and the exact gelu, and of layers with a norm on either side of every branch."""
 
 from __future__ import annotations
@@ -42,59 +43,94 @@ def _pairs(x, ids, n_experts):
         raise KernelError("routed experts: a negative number of experts")
 
 
-def expert_glu_pairs(x: torch.Tensor, w_gate_up: torch.Tensor, ids: torch.Tensor) -> torch.Tensor:
-    """``mid[t, j] = silu(Wg[e] x[t]) * (Wu[e] x[t])`` with ``e = ids[t, j]``, for every pair whose ``e`` is below
-    the number of experts ``w_gate_up`` [E, 2F, D] holds (gate rows, then up rows); the others are left unwritten.
-    Returns [n, top, F] of x's dtype."""
-    _gpu(x, w_gate_up, ids)
-    E = w_gate_up.shape[0] if w_gate_up.dim() == 3 else -1
-    _pairs(x, ids, E)
-    n, D = x.shape
-    if w_gate_up.dim() != 3 or w_gate_up.shape[2] != D or w_gate_up.shape[1] % 2 or w_gate_up.dtype != x.dtype or not w_gate_up.is_contiguous():
-        raise KernelError(f"expert_glu_pairs: weights must be contiguous [E, 2F, {D}] of x's dtype")
-    F = w_gate_up.shape[1] // 2
-    top = ids.shape[1]
-    mid = torch.empty((n, top, F), dtype=x.dtype, device=x.device)
-    check(core().tl_expert_glu_pairs(x.data_ptr(), w_gate_up.data_ptr(), ids.data_ptr(), top, E, mid.data_ptr(), n, D, F,
-                                     dtype_code(x.dtype), _stream()))
+def _expert_rows(rows, weights, offsets, what):
+    if rows.dim() != 2 or not rows.is_contiguous():
+        raise KernelError(f"{what}: the rows must be a contiguous matrix")
+    if weights.dim() != 3 or weights.shape[2] != rows.shape[1] or weights.dtype != rows.dtype or not weights.is_contiguous():
+        raise KernelError(f"{what}: weights must be contiguous [E, outputs, {rows.shape[1]}] of the rows' dtype")
+    if offsets.dtype != torch.int32 or offsets.dim() != 1 or offsets.numel() < weights.shape[0] + 1 or not offsets.is_contiguous():
+        raise KernelError(f"{what}: offsets must be contiguous int32 with an entry per expert and one more")
+
+
+def expert_glu_rows(rows: torch.Tensor, w_gate_up: torch.Tensor, offsets: torch.Tensor) -> torch.Tensor:
+    """``mid[r] = silu(Wg[e] rows[r]) * (Wu[e] rows[r])`` for the rows ``offsets[e] .. offsets[e + 1]`` of every expert
+    ``e`` of ``w_gate_up`` [E, 2F, D] (gate rows, then up rows); ``rows`` [pairs, D] as ``expert_gather`` leaves them.
+    An expert's weights are read once for up to eight of its rows.  Returns [pairs, F]; rows behind ``offsets[E]`` (pairs of
+    outputs that are no experts) are left unwritten."""
+    _gpu(rows, w_gate_up, offsets)
+    _expert_rows(rows, w_gate_up, offsets, "expert_glu_rows")
+    if w_gate_up.shape[1] % 2:
+        raise KernelError("expert_glu_rows: gate rows and up rows of every expert")
+    E, F, D = w_gate_up.shape[0], w_gate_up.shape[1] // 2, rows.shape[1]
+    mid = torch.empty((rows.shape[0], F), dtype=rows.dtype, device=rows.device)
+    check(core().tl_expert_glu_rows(rows.data_ptr(), w_gate_up.data_ptr(), offsets.data_ptr(), E, mid.data_ptr(), D, F,
+                                    rows.shape[0], dtype_code(rows.dtype), _stream()))
     return mid
 
 
-def expert_down_pairs(
-    mid: torch.Tensor,
-    w_down: torch.Tensor,
+def expert_down_rows(mid: torch.Tensor, w_down: torch.Tensor, offsets: torch.Tensor) -> torch.Tensor:
+    """``y[r] = Wd[e] mid[r]`` in 32-bit for the rows ``offsets[e] .. offsets[e + 1]`` of every expert of ``w_down``
+    [E, D, F].  Returns float32 [pairs, D]."""
+    _gpu(mid, w_down, offsets)
+    _expert_rows(mid, w_down, offsets, "expert_down_rows")
+    E, D, F = w_down.shape
+    y = torch.empty((mid.shape[0], D), dtype=torch.float32, device=mid.device)
+    check(core().tl_expert_down_rows(mid.data_ptr(), w_down.data_ptr(), offsets.data_ptr(), E, y.data_ptr(), D, F,
+                                     mid.shape[0], dtype_code(mid.dtype), _stream()))
+    return y
+
+
+def expert_gather(x: torch.Tensor, ids: torch.Tensor, n_out: int):
+    """The (token, choice) pairs in the order of their experts.  Returns ``(rows, pos, offsets)``: ``rows`` [n * top, D]
+    holds for every pair its token's row of ``x``, the pairs of output e in the rows ``offsets[e] .. offsets[e + 1]``
+    (int32 [n_out + 1], on the device); ``pos`` int32 [n, top] says which row each pair got."""
+    _gpu(x, ids)
+    _pairs(x, ids, 0)
+    n, D = x.shape
+    top = ids.shape[1]
+    work = torch.zeros(3 * n_out + 1, dtype=torch.int32, device=x.device)
+    counts, offsets, cursor = work[:n_out], work[n_out : 2 * n_out + 1], work[2 * n_out + 1 :]
+    pos = torch.empty((n, top), dtype=torch.int32, device=x.device)
+    rows = torch.empty((n * top, D), dtype=x.dtype, device=x.device)
+    check(core().tl_expert_gather(x.data_ptr(), ids.data_ptr(), n, top, n_out, counts.data_ptr(), offsets.data_ptr(), cursor.data_ptr(),
+                                  pos.data_ptr(), rows.data_ptr(), D, dtype_code(x.dtype), _stream()))
+    return rows, pos, offsets
+
+
+def expert_combine(
+    y: torch.Tensor,
+    pos: torch.Tensor,
     ids: torch.Tensor,
     weights: torch.Tensor,
+    n_experts: int,
     x: torch.Tensor,
     shared: Optional[torch.Tensor] = None,
     shared_gate: Optional[torch.Tensor] = None,
 ) -> torch.Tensor:
-    """``out[t] = sum_j weights[t, j] * (Wd[e] mid[t, j] if e = ids[t, j] is an expert of w_down [E, D, F], else x[t])``,
-    plus ``sigmoid(shared_gate[t]) * shared[t]`` when a shared expert's result [n, D] and its gate's 32-bit
-    pre-activation (one number a token: a column of some matrix will do) are given.  Returns [n, D] of x's dtype."""
-    _gpu(mid, w_down, ids, weights, x, shared, shared_gate)
-    E = w_down.shape[0] if w_down.dim() == 3 else -1
-    _pairs(x, ids, E)
+    """``out[t] = sum_j weights[t, j] * (y[pos[t, j]] if ids[t, j] < n_experts else x[t])``, plus
+    ``sigmoid(shared_gate[t]) * shared[t]``: the experts' results (rows in the order ``expert_gather`` gave them) back
+    in the order of the tokens; ``y`` is 32-bit (``expert_down_rows``) or of x's dtype (matrix products over the
+    gathered rows).  Returns [n, D] of x's dtype."""
+    _gpu(y, pos, ids, weights, x, shared, shared_gate)
+    _pairs(x, ids, n_experts)
     n, D = x.shape
     top = ids.shape[1]
-    if w_down.dim() != 3 or w_down.shape[1] != D or w_down.dtype != x.dtype or not w_down.is_contiguous():
-        raise KernelError(f"expert_down_pairs: weights must be contiguous [E, {D}, F] of x's dtype")
-    F = w_down.shape[2]
-    if tuple(mid.shape) != (n, top, F) or mid.dtype != x.dtype or not mid.is_contiguous():
-        raise KernelError(f"expert_down_pairs: mid must be contiguous [{n}, {top}, {F}] of x's dtype")
+    if y.dim() != 2 or y.shape[1] != D or y.dtype not in (x.dtype, torch.float32) or not y.is_contiguous():
+        raise KernelError("expert_combine: y must be a contiguous [rows, D] matrix of x's dtype or of float32")
+    if tuple(pos.shape) != (n, top) or pos.dtype != torch.int32 or not pos.is_contiguous():
+        raise KernelError("expert_combine: pos must be contiguous int32 [n, top]")
     if tuple(weights.shape) != (n, top) or weights.dtype != torch.float32 or not weights.is_contiguous():
-        raise KernelError("expert_down_pairs: weights must be contiguous float32 [n, top]")
+        raise KernelError("expert_combine: weights must be contiguous float32 [n, top]")
     sg_stride = 0
     if shared is not None:
         if tuple(shared.shape) != (n, D) or shared.dtype != x.dtype or not shared.is_contiguous():
-            raise KernelError("expert_down_pairs: the shared expert's result must be contiguous [n, D] of x's dtype")
+            raise KernelError("expert_combine: the shared expert's result must be contiguous [n, D] of x's dtype")
         if shared_gate is None or shared_gate.dtype != torch.float32 or shared_gate.numel() != n or shared_gate.dim() > 2:
-            raise KernelError("expert_down_pairs: the shared expert's gate must be float32, one number a token")
+            raise KernelError("expert_combine: the shared expert's gate must be float32, one number a token")
         sg_stride = shared_gate.stride(0) if n > 1 else 1
     out = torch.empty((n, D), dtype=x.dtype, device=x.device)
-    check(core().tl_expert_down_pairs(mid.data_ptr(), w_down.data_ptr(), ids.data_ptr(), weights.data_ptr(), top, E, x.data_ptr(),
-                                      _ptr(shared), _ptr(shared_gate), sg_stride, out.data_ptr(), n, D, F, dtype_code(x.dtype),
-                                      _stream()))
+    check(core().tl_expert_combine(y.data_ptr(), 1 if y.dtype == torch.float32 else 0, pos.data_ptr(), ids.data_ptr(), weights.data_ptr(), top, n_experts, x.data_ptr(),
+                                   _ptr(shared), _ptr(shared_gate), sg_stride, out.data_ptr(), n, D, dtype_code(x.dtype), _stream()))
     return out
 
 

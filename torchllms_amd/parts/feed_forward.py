@@ -79,10 +79,16 @@ class RoutedExperts(FeedForward):
     chosen experts' outputs times their ``s`` (not renormalised).  ``shared_size`` f > 0: an expert of that width runs
     for every token and is added times ``sigmoid(W_sg x)``, one number a token.
 
-    A token's result depends on nothing but the token.  Every (token, choice) is worked on by itself, whatever the
-    step's shape, so a decode step's launches are fixed by its shape."""
+    A token's result depends on nothing but the token.  The (token, choice) pairs of a step are put in the order of
+    their experts on the device, and a kernel walks every expert's rows with the expert's weights read once for eight
+    of them; each row's sums have an order of their own, so in 32-bit a token's result has the same bits in every
+    step, and the launches are fixed by the step's shape (decode steps are replayed from graphs).  A bfloat16 step
+    that brings prompts and has ``GROUPED_FROM`` pairs or more runs one matrix product per expert over its rows
+    instead; for that the host reads how many rows each expert got, once a layer."""
 
     graph_safe = True
+    #: (token, choice) pairs of a bfloat16 step with prompts from which on the experts run as matrix products
+    GROUPED_FROM = 512
 
     def __init__(self, hidden_size: int, expert_size: int, num_experts: int, top: int, num_identity: int = 0, shared_size: int = 0):
         for name, v in (("expert_size", expert_size), ("num_experts", num_experts), ("top", top)):
@@ -134,9 +140,20 @@ class RoutedExperts(FeedForward):
         n_out = self.E + self.I
         z = ops.linear(x, self.w_router, out_dtype=torch.float32)
         ids, weights = ops.router_topk(z, n_out, self.correction, self.top)
-        mid = ops.expert_glu_pairs(x, self.w_gu, ids)
         shared = gate = None
         if self.shared:
             shared = ops.linear(ops.linear_glu(x, self.shared_w13), self.shared_w2)
             gate = z[:, n_out]
-        return ops.expert_down_pairs(mid, self.w_down, ids, weights, x, shared, gate)
+        rows, pos, offsets = ops.expert_gather(x, ids, n_out)
+        if x.dtype == torch.float32 or ctx.host.max_q_len <= 1 or x.shape[0] * self.top < self.GROUPED_FROM:
+            y = ops.expert_down_rows(ops.expert_glu_rows(rows, self.w_gu, offsets), self.w_down, offsets)
+            return ops.expert_combine(y, pos, ids, weights, self.E, x, shared, gate)
+        bounds = offsets.tolist()  # (the one place a step with prompts waits for the GPU)
+        parts = []
+        for e in range(self.E):
+            lo, hi = bounds[e], bounds[e + 1]
+            if hi > lo:
+                parts.append(ops.linear(ops.linear_glu(rows[lo:hi], self.w_gu[e]), self.w_down[e]))
+        # (the rows of experts that hand their input through lie behind all others and are never read)
+        y = torch.cat(parts) if parts else rows
+        return ops.expert_combine(y, pos, ids, weights, self.E, x, shared, gate)
