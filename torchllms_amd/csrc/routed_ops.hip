@@ -391,6 +391,59 @@ post_norm_add_norm_kernel(float* __restrict__ stream, const T* __restrict__ y, c
   for (int i = threadIdx.x; i < hidden; i += kSandwichThreads) rows[r * hidden + i] = from_f32<T>(row_l[i] * inv2 * w_next[i]);
 }
 
+
+// The same for few rows of up to HELD * 256 elements: a launch is then as long as a row's trips to memory, so everything
+// a thread needs is asked for at once (an element past the end is the row's first once more, and not used).  Operation
+// for operation the kernel above: the same bits.
+template <typename T, int HELD>
+__global__ void __launch_bounds__(kSandwichThreads)
+post_norm_add_norm_held_kernel(float* __restrict__ stream, const T* __restrict__ y, const float* __restrict__ w_post, float eps,
+                               const float* __restrict__ w_next, float eps_next, T* __restrict__ rows, int hidden) {
+#pragma clang fp contract(off)
+  __shared__ float scratch[kSandwichThreads / kWave];
+  const size_t r = blockIdx.x;
+  const T* yr = y + r * hidden;
+  float* sr = stream + r * hidden;
+  T yraw[HELD];
+  float sv[HELD], wp[HELD], wn[HELD];
+#pragma unroll
+  for (int c = 0; c < HELD; ++c) {
+    const int i = threadIdx.x + c * kSandwichThreads;
+    const int at = i < hidden ? i : 0;
+    yraw[c] = yr[at];
+    sv[c] = sr[at];
+    wp[c] = w_post[at];
+    wn[c] = w_next ? w_next[at] : 0.f;
+  }
+  float yv[HELD];
+  float ss = 0.f;
+#pragma unroll
+  for (int c = 0; c < HELD; ++c) {
+    yv[c] = threadIdx.x + c * kSandwichThreads < hidden ? to_f32(yraw[c]) : 0.f;
+    ss += yv[c] * yv[c];
+  }
+  ss = block_sum<kSandwichThreads / kWave>(ss, scratch);
+  const float inv = 1.0f / sqrtf(ss / (float)hidden + eps);
+  float s2 = 0.f;
+#pragma unroll
+  for (int c = 0; c < HELD; ++c) {
+    const int i = threadIdx.x + c * kSandwichThreads;
+    if (i < hidden) {
+      sv[c] = sv[c] + yv[c] * inv * wp[c];
+      sr[i] = sv[c];
+      s2 += sv[c] * sv[c];
+    }
+  }
+  if (w_next == nullptr) return;
+  s2 = block_sum<kSandwichThreads / kWave>(s2, scratch);
+  const float inv2 = 1.0f / sqrtf(s2 / (float)hidden + eps_next);
+#pragma unroll
+  for (int c = 0; c < HELD; ++c) {
+    const int i = threadIdx.x + c * kSandwichThreads;
+    if (i < hidden) rows[r * hidden + i] = from_f32<T>(sv[c] * inv2 * wn[c]);
+  }
+}
+
 }  // namespace
 
 // ============================================================================= C interface
@@ -541,12 +594,19 @@ TL_EXPORT int tl_post_norm_add_norm(float* stream_rows, const void* y, const flo
   const size_t lds = (size_t)hidden * sizeof(float);
   if (lds + 64 > (size_t)tl_device_facts().lds_bytes)
     return tl_fail(TL_ERR_UNSUPPORTED, "post_norm_add_norm: rows of %d elements do not fit the LDS", hidden);
-  if (dtype == TL_F32)
-    post_norm_add_norm_kernel<float><<<n, kSandwichThreads, lds, stream>>>(stream_rows, (const float*)y, w_post, eps, w_next, eps_next,
-                                                                         (float*)rows, hidden);
-  else if (dtype == TL_BF16)
-    post_norm_add_norm_kernel<bf16_t><<<n, kSandwichThreads, lds, stream>>>(stream_rows, (const bf16_t*)y, w_post, eps, w_next, eps_next,
-                                                                          (bf16_t*)rows, hidden);
-  else return tl_fail(TL_ERR_ARG, "post_norm_add_norm: unknown dtype %d", dtype);
+  if (dtype != TL_F32 && dtype != TL_BF16) return tl_fail(TL_ERR_ARG, "post_norm_add_norm: unknown dtype %d", dtype);
+  const bool few = n <= 2 * tl_device_facts().compute_units;
+#define TL_SANDWICH(T)                                                                                                         \
+  do {                                                                                                                         \
+    if (few && hidden <= 4 * kSandwichThreads)                                                                                 \
+      post_norm_add_norm_held_kernel<T, 4><<<n, kSandwichThreads, 0, stream>>>(stream_rows, (const T*)y, w_post, eps, w_next, eps_next, (T*)rows, hidden);  \
+    else if (few && hidden <= 16 * kSandwichThreads)                                                                           \
+      post_norm_add_norm_held_kernel<T, 16><<<n, kSandwichThreads, 0, stream>>>(stream_rows, (const T*)y, w_post, eps, w_next, eps_next, (T*)rows, hidden); \
+    else                                                                                                                       \
+      post_norm_add_norm_kernel<T><<<n, kSandwichThreads, lds, stream>>>(stream_rows, (const T*)y, w_post, eps, w_next, eps_next, (T*)rows, hidden);        \
+  } while (0)
+  if (dtype == TL_F32) TL_SANDWICH(float);
+  else TL_SANDWICH(bf16_t);
+#undef TL_SANDWICH
   return tl_check_launch("post_norm_add_norm");
 }

@@ -781,6 +781,12 @@ gated_delta_step_kernel(const T* __restrict__ qkv, int qkv_stride, const T* __re
     const int dd = d < dk ? d : d - dk;
     (d < dk ? k_l : q_l)[dd + dd / 16 * 4] = to_f32(tok[d < dk ? G * dk + g * dk + dd : g * dk + dd]);
   }
+  float* g_l = lds + 2 * dkp;  // (CH) the token's decays, once for all columns of the block
+  if (CH) {
+    const float rate = -expf(A_log[h]);
+    for (int d = threadIdx.x; d < dk; d += blockDim.x)
+      g_l[d + d / 16 * 4] = expf(rate * softplus_f(a_ch[t * a_stride + h * dk + d] + dt_bias[h * dk + d]));
+  }
   float* st = state + (long long)slot_ids[row] * state_stride + ((size_t)h * dv + j) * dk;
   float S[kDeltaRows];
   if (VEC) {
@@ -820,7 +826,7 @@ gated_delta_step_kernel(const T* __restrict__ qkv, int qkv_stride, const T* __re
     kk[r] = in ? k_l[i + i / 16 * 4] * k_inv : 0.f;
     const float qq = in ? q_l[i + i / 16 * 4] * q_inv : 0.f;
     float dec = decay;
-    if (CH) dec = in ? expf(neg_rate * softplus_f(a_ch[t * a_stride + h * dk + i] + dt_bias[h * dk + i])) : 0.f;
+    if (CH) dec = in ? g_l[i + i / 16 * 4] : 0.f;
     S[r] = dec * S[r];
     kv[r % 4] = fmaf(S[r], kk[r], kv[r % 4]);
     sq[r % 4] = fmaf(S[r], qq, sq[r % 4]);
@@ -1125,7 +1131,7 @@ TL_EXPORT int tl_gated_delta(const void* qkv, int qkv_stride, const void* proj, 
   const bool vec = dk % 4 == 0 && ((uintptr_t)state % 16) == 0 && state_stride % 4 == 0;
 #define TL_DELTA_STEP(T, VEC, CH)                                                                                      \
   do {                                                                                                                 \
-    const size_t step_lds = 2 * (size_t)dkp * sizeof(float);                                                           \
+    const size_t step_lds = (CH ? 3 : 2) * (size_t)dkp * sizeof(float);                                               \
     if (rows == 8)                                                                                                     \
       gated_delta_step_kernel<T, VEC, 8, CH><<<grid, threads, step_lds, stream>>>(                                     \
           (const T*)qkv, qkv_stride, (const T*)proj, proj_stride, b_off, a_off, A_log, dt_bias, state, state_stride,   \
