@@ -253,9 +253,85 @@ expert_rows_held_kernel(const bf16_t* __restrict__ rows, const bf16_t* __restric
   }
 }
 
+// The same two products on the matrix cores, for experts with many rows: a wave takes 16 outputs of one expert and up
+// to 32 of its rows at a time, and walks K in steps of 128: a lane asks for four neighbouring 16-byte pieces of its
+// weight row (and of its up row) and of its one or two rows of x, straight from memory (the rows are small and come from
+// the caches; no LDS, no barrier), and every piece is one MFMA 16x16x32 (which k a lane holds does not matter as long as
+// both operands hold the same).  acc[i] = C[row 16 c + lane % 16][output n0 + 4 (lane / 16) + i].
+typedef float float4_r __attribute__((ext_vector_type(4)));
+constexpr int kRowsMfmaFrom = 8;  // pairs of a step above which the experts' products run on the matrix cores
+template <bool GLU>
+__global__ void __launch_bounds__(kRowsThreads)
+expert_rows_mfma_kernel(const bf16_t* __restrict__ rows, const bf16_t* __restrict__ w, const int32_t* __restrict__ offsets,
+                        bf16_t* __restrict__ mid, float* __restrict__ y, int K, int N) {
+  const int e = blockIdx.x;
+  const int lo = offsets[e], hi = offsets[e + 1];
+  if (lo == hi) return;
+  const int wave = threadIdx.x / kWave, lane = threadIdx.x % kWave;
+  const int n16 = lane & 15, g4 = lane >> 4;
+  const int n0 = (blockIdx.y * (kRowsThreads / kWave) + wave) * 16;
+  if (n0 >= N) return;
+  const int n_mine = n0 + n16 < N ? n0 + n16 : N - 1;
+  const bf16_t* g_row = w + ((size_t)e * (GLU ? 2 : 1) * N + n_mine) * K;
+  const bf16_t* u_row = g_row + (size_t)N * K;
+  bf16x8_r zero;
+#pragma unroll
+  for (int i = 0; i < 8; ++i) zero[i] = (__bf16)0.0f;
+  for (int r0 = lo; r0 < hi; r0 += 32) {
+    const bool two = r0 + 16 < hi;
+    const bf16_t* x0 = rows + (size_t)min(r0 + n16, hi - 1) * K;
+    const bf16_t* x1 = rows + (size_t)min(r0 + 16 + n16, hi - 1) * K;
+    float4_r ag0 = {0.f, 0.f, 0.f, 0.f}, ag1 = ag0, au0 = ag0, au1 = ag0;
+    for (int k0 = 0; k0 < K; k0 += 128) {
+      bf16x8_r gw[4], uw[4], xa[4], xb[4];
+#pragma unroll
+      for (int u = 0; u < 4; ++u) {
+        const int kk = k0 + 8 * (4 * g4 + u);
+        const bool in = kk < K;
+        const int at = in ? kk : 0;
+        gw[u] = *reinterpret_cast<const bf16x8_r*>(g_row + at);
+        if (GLU) uw[u] = *reinterpret_cast<const bf16x8_r*>(u_row + at);
+        xa[u] = *reinterpret_cast<const bf16x8_r*>(x0 + at);
+        if (two) xb[u] = *reinterpret_cast<const bf16x8_r*>(x1 + at);
+        if (!in) { xa[u] = zero; xb[u] = zero; }
+      }
+#pragma unroll
+      for (int u = 0; u < 4; ++u) {
+        ag0 = __builtin_amdgcn_mfma_f32_16x16x32_bf16(gw[u], xa[u], ag0, 0, 0, 0);
+        if (GLU) au0 = __builtin_amdgcn_mfma_f32_16x16x32_bf16(uw[u], xa[u], au0, 0, 0, 0);
+        if (two) {
+          ag1 = __builtin_amdgcn_mfma_f32_16x16x32_bf16(gw[u], xb[u], ag1, 0, 0, 0);
+          if (GLU) au1 = __builtin_amdgcn_mfma_f32_16x16x32_bf16(uw[u], xb[u], au1, 0, 0, 0);
+        }
+      }
+    }
+#pragma unroll
+    for (int c = 0; c < 2; ++c) {
+      const int r = r0 + 16 * c + n16;
+      if (r < hi && (c == 0 || two)) {
+        const float4_r g = c == 0 ? ag0 : ag1, uu = c == 0 ? au0 : au1;
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+          const int n = n0 + 4 * g4 + i;
+          if (n < N) {
+            if (GLU) mid[(size_t)r * N + n] = from_f32<bf16_t>(silu_r(g[i]) * uu[i]);
+            else y[(size_t)r * N + n] = g[i];
+          }
+        }
+      }
+    }
+  }
+}
+
 template <bool GLU>
 static int launch_rows_held(const void* rows, const void* w, const int32_t* offsets, int n_experts, void* mid, float* y, int K, int N,
                             int max_rows, hipStream_t stream) {
+  if (max_rows > kRowsMfmaFrom) {
+    // more rows than a few: the matrix cores (an expert can have that many; one that has not pays little for it)
+    const dim3 mgrid(n_experts, (N + 16 * (kRowsThreads / kWave) - 1) / (16 * (kRowsThreads / kWave)));
+    expert_rows_mfma_kernel<GLU><<<mgrid, kRowsThreads, 0, stream>>>((const bf16_t*)rows, (const bf16_t*)w, offsets, (bf16_t*)mid, y, K, N);
+    return tl_check_launch("expert_rows_mfma");
+  }
   int at_once = 1;
   while (at_once < kHeldRows && at_once < max_rows) at_once *= 2;
   while (at_once > 1 && (size_t)at_once * K * 2 > 32 * 1024) at_once /= 2;
