@@ -1378,6 +1378,86 @@ matrix_memory_kernel(const T* __restrict__ proj, int stride, int q_off, int k_of
     if (part == 0) *m_at = sc_l[4 * kDeltaTile];
   }
 }
+
+// The same cell for a step in which every request brings one token (decode): no tiles, nothing fetched ahead, every
+// thread works the gates out for itself.  Every product and sum is taken as matrix_memory_kernel takes it, so a token's
+// result has the same bits from either kernel.
+template <typename T, bool VEC, int R>
+__global__ void __launch_bounds__(512)
+matrix_memory_step_kernel(const T* __restrict__ proj, int stride, int q_off, int k_off, int v_off, int i_off, int f_off,
+                          const float* __restrict__ i_bias, const float* __restrict__ f_bias, float cap,
+                          float* __restrict__ state, long long state_stride, const int32_t* __restrict__ qo_indptr,
+                          const int32_t* __restrict__ slot_ids, float* __restrict__ o_raw, float* __restrict__ den, int H,
+                          int dk, int dv, int lpc, int col_groups) {
+  extern __shared__ __attribute__((aligned(16))) float lds[];
+  const int dkp = dk + dk / 16 * 4;
+  float* k_l = lds;
+  float* q_l = lds + dkp;
+  const int W = dv + 1;
+  const int row = blockIdx.y;
+  const int h = blockIdx.x / col_groups, cg = blockIdx.x % col_groups;
+  const size_t t = (size_t)qo_indptr[row];
+  const int j_loc = threadIdx.x / lpc, part = threadIdx.x % lpc;
+  const int j_raw = cg * kMemCols + j_loc;
+  const bool live = j_loc < kMemCols && j_raw < W;
+  const int j = j_raw < W ? j_raw : W - 1;
+  const bool norm_col = j == dv;
+  const int i0 = part * R;
+  float* slot = state + (long long)slot_ids[row] * state_stride;
+  float* st = slot + ((size_t)h * W + j) * dk;
+  float* m_at = slot + (size_t)H * W * dk + (size_t)h * W + j;
+  const T* tok = proj + t * stride;
+  const float m = *m_at;
+  const float gi = cap * tanhf((to_f32(tok[i_off + h]) + i_bias[h]) / cap);
+  const float gf = log_sigmoid_f(cap * tanhf((to_f32(tok[f_off + h]) + f_bias[h]) / cap));
+  const float m_new = fmaxf(gf + m, gi);
+  const float keep = expf(gf + m - m_new), take = expf(gi - m_new), floor = expf(-m_new);
+  const float q_scale = 1.0f / sqrtf((float)dk);
+  for (int d = threadIdx.x; d < 2 * dk; d += blockDim.x) {
+    const int dd = d < dk ? d : d - dk;
+    (d < dk ? k_l : q_l)[dd + dd / 16 * 4] = to_f32(tok[d < dk ? k_off + h * dk + dd : q_off + h * dk + dd]) * (d < dk ? take : q_scale);
+  }
+  float S[R];
+  if (VEC) {
+#pragma unroll
+    for (int r = 0; r < R; r += 4) {
+      const float4 s4 = i0 + r < dk ? *reinterpret_cast<const float4*>(st + i0 + r) : float4{0.f, 0.f, 0.f, 0.f};
+      S[r] = s4.x; S[r + 1] = s4.y; S[r + 2] = s4.z; S[r + 3] = s4.w;
+    }
+  } else {
+#pragma unroll
+    for (int r = 0; r < R; ++r) S[r] = i0 + r < dk ? st[i0 + r] : 0.f;
+  }
+  const float v = norm_col ? 1.0f : to_f32(tok[v_off + h * dv + j]);
+  __syncthreads();
+  float sq[4] = {0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+  for (int r = 0; r < R; ++r) {
+    const int i = i0 + r;
+    const bool in = i < dk;
+    const float kk = in ? k_l[i + i / 16 * 4] : 0.f;
+    const float qq = in ? q_l[i + i / 16 * 4] : 0.f;
+    S[r] = fmaf(kk, v, keep * S[r]);
+    sq[r % 4] = fmaf(S[r], qq, sq[r % 4]);
+  }
+  const float sq_all = row_group_sum((sq[0] + sq[1]) + (sq[2] + sq[3]), lpc);
+  if (live && part == 0) {
+    if (norm_col) den[t * H + h] = fmaxf(fabsf(sq_all), floor) + 1e-6f;
+    else o_raw[(t * H + h) * dv + j] = sq_all;
+  }
+  if (live) {
+    if (VEC) {
+#pragma unroll
+      for (int r = 0; r < R; r += 4)
+        if (i0 + r < dk) *reinterpret_cast<float4*>(st + i0 + r) = float4{S[r], S[r + 1], S[r + 2], S[r + 3]};
+    } else {
+#pragma unroll
+      for (int r = 0; r < R; ++r)
+        if (i0 + r < dk) st[i0 + r] = S[r];
+    }
+    if (part == 0) *m_at = m_new;
+  }
+}
 }  // namespace
 
 // proj [n_tokens, stride]: the columns of q (H * dk from q_off), k, v (H * dv) and of the two gates' pre-activations
@@ -1404,10 +1484,19 @@ TL_EXPORT int tl_matrix_memory(const void* proj, int stride, int q_off, int k_of
   const size_t lds = ((size_t)kDeltaTile * (2 * dkp + 2 * kMemCols + 4) + 4) * sizeof(float);
   const dim3 grid(H * col_groups, n_seqs);
   const bool vec = dk % 4 == 0 && ((uintptr_t)state % 16) == 0 && state_stride % 4 == 0;
+  const bool single = n_tokens == n_seqs;
+  const size_t step_lds = 2 * (size_t)dkp * sizeof(float);
 #define TL_MEM(T, VEC, R)                                                                                               \
-  matrix_memory_kernel<T, VEC, R><<<grid, threads, lds, stream>>>((const T*)proj, stride, q_off, k_off, v_off, i_off, f_off, \
-                                                                  i_bias, f_bias, cap, state, state_stride, qo_indptr,  \
-                                                                  slot_ids, o_raw, den, H, dk, dv, lpc, col_groups)
+  do {                                                                                                                  \
+    if (single)                                                                                                         \
+      matrix_memory_step_kernel<T, VEC, R><<<grid, threads, step_lds, stream>>>(                                        \
+          (const T*)proj, stride, q_off, k_off, v_off, i_off, f_off, i_bias, f_bias, cap, state, state_stride, qo_indptr, \
+          slot_ids, o_raw, den, H, dk, dv, lpc, col_groups);                                                            \
+    else                                                                                                                \
+      matrix_memory_kernel<T, VEC, R><<<grid, threads, lds, stream>>>(                                                  \
+          (const T*)proj, stride, q_off, k_off, v_off, i_off, f_off, i_bias, f_bias, cap, state, state_stride, qo_indptr, \
+          slot_ids, o_raw, den, H, dk, dv, lpc, col_groups);                                                            \
+  } while (0)
 #define TL_MEM_T(T)                                  \
   do {                                               \
     if (vec && rows == 8) TL_MEM(T, true, 8);        \
