@@ -353,39 +353,47 @@ def test_router_kernel_and_experts_against_the_plain_functions():
         assert torch.allclose(wts.cpu().double(), s.gather(1, ids.cpu().long()), atol=1e-6)
         plain_choice = torch.topk(s, top).indices.sort(-1).values
         assert n_out == top or not torch.equal(plain_choice, want_ids.sort(-1).values)  # the correction matters
-    n, D, F, E, I, top = 61, 48, 40, 4, 2, 3
-    x = torch.randn((n, D), generator=g)
-    w_gu = torch.randn((E, 2 * F, D), generator=g) * 0.2
-    w_d = torch.randn((E, D, F), generator=g) * 0.2
-    ids = torch.stack([torch.randperm(E + I, generator=g)[:top] for _ in range(n)]).to(torch.int32)
-    wts = torch.rand((n, top), generator=g)
-    shared, sg = torch.randn((n, D), generator=g), torch.randn((n, 3), generator=g)
-    for dtype, tol in ((torch.float32, 1e-5), (torch.bfloat16, 3e-2)):
-        xd = x.to(dtype).to(dev)
-        rows, pos, offsets = ops.expert_gather(xd, ids.to(dev), E + I)
-        y = ops.expert_down_rows(ops.expert_glu_rows(rows, w_gu.to(dtype).to(dev), offsets), w_d.to(dtype).to(dev), offsets)
-        got = ops.expert_combine(y, pos, ids.to(dev), wts.to(dev), E, xd, shared.to(dtype).to(dev), sg.to(dev)[:, 1])
-        xr, gu, dn, sh = x.to(dtype).double(), w_gu.to(dtype).double(), w_d.to(dtype).double(), shared.to(dtype).double()
-        want = plain.sigmoid(sg[:, 1:2].double()) * sh
-        for t in range(n):
-            for j in range(top):
-                e = int(ids[t, j])
-                y = xr[t] if e >= E else dn[e] @ (plain.silu(gu[e, :F] @ xr[t]) * (gu[e, F:] @ xr[t]))
-                want[t] += float(wts[t, j]) * y
-        assert (got.double().cpu() - want).abs().max() < tol * want.abs().max()
-        # the gathered rows themselves, and the same result through one matrix product per expert
-        bounds = offsets.tolist()
-        assert bounds[0] == 0 and bounds[-1] == n * top
-        assert [bounds[e + 1] - bounds[e] for e in range(E + I)] == torch.bincount(ids.flatten().long(), minlength=E + I).tolist()
-        assert sorted(pos.flatten().tolist()) == list(range(n * top))
-        for t in range(n):
-            for j in range(top):
-                at = int(pos[t, j])
-                assert bounds[int(ids[t, j])] <= at < bounds[int(ids[t, j]) + 1] and torch.equal(rows[at], xd[t])
-        parts = [ops.linear(ops.linear_glu(rows[bounds[e] : bounds[e + 1]], w_gu.to(dtype).to(dev)[e]), w_d.to(dtype).to(dev)[e])
-                 for e in range(E) if bounds[e + 1] > bounds[e]]
-        again = ops.expert_combine(torch.cat(parts), pos, ids.to(dev), wts.to(dev), E, xd, shared.to(dtype).to(dev), sg.to(dev)[:, 1])
-        assert (again.double().cpu() - want).abs().max() < 2 * tol * want.abs().max()
+    # (many pairs: the matrix cores; few: a wave an output with its weights in registers)
+    for n in (61, 2):
+        D, F, E, I, top = 48, 40, 4, 2, 3
+        x = torch.randn((n, D), generator=g)
+        w_gu = torch.randn((E, 2 * F, D), generator=g) * 0.2
+        w_d = torch.randn((E, D, F), generator=g) * 0.2
+        ids = torch.stack([torch.randperm(E + I, generator=g)[:top] for _ in range(n)]).to(torch.int32)
+        wts = torch.rand((n, top), generator=g)
+        shared, sg = torch.randn((n, D), generator=g), torch.randn((n, 3), generator=g)
+        for dtype, tol in ((torch.float32, 1e-5), (torch.bfloat16, 3e-2)):
+            xd = x.to(dtype).to(dev)
+            rows, pos, offsets = ops.expert_gather(xd, ids.to(dev), E + I)
+            y = ops.expert_down_rows(ops.expert_glu_rows(rows, w_gu.to(dtype).to(dev), offsets), w_d.to(dtype).to(dev), offsets)
+            got = ops.expert_combine(y, pos, ids.to(dev), wts.to(dev), E, xd, shared.to(dtype).to(dev), sg.to(dev)[:, 1])
+            xr, gu, dn, sh = x.to(dtype).double(), w_gu.to(dtype).double(), w_d.to(dtype).double(), shared.to(dtype).double()
+            want = plain.sigmoid(sg[:, 1:2].double()) * sh
+            for t in range(n):
+                for j in range(top):
+                    e = int(ids[t, j])
+                    y = xr[t] if e >= E else dn[e] @ (plain.silu(gu[e, :F] @ xr[t]) * (gu[e, F:] @ xr[t]))
+                    want[t] += float(wts[t, j]) * y
+            assert (got.double().cpu() - want).abs().max() < tol * want.abs().max()
+            # the gathered rows themselves, and the same result through one matrix product per expert
+            bounds = offsets.tolist()
+            assert bounds[0] == 0 and bounds[-1] == n * top
+            assert [bounds[e + 1] - bounds[e] for e in range(E + I)] == torch.bincount(ids.flatten().long(), minlength=E + I).tolist()
+            assert sorted(pos.flatten().tolist()) == list(range(n * top))
+            for t in range(n):
+                for j in range(top):
+                    at = int(pos[t, j])
+                    assert bounds[int(ids[t, j])] <= at < bounds[int(ids[t, j]) + 1] and torch.equal(rows[at], xd[t])
+            parts = [ops.linear(ops.linear_glu(rows[bounds[e] : bounds[e + 1]], w_gu.to(dtype).to(dev)[e]), w_d.to(dtype).to(dev)[e])
+                     for e in range(E) if bounds[e + 1] > bounds[e]]
+            again = ops.expert_combine(torch.cat(parts), pos, ids.to(dev), wts.to(dev), E, xd, shared.to(dtype).to(dev), sg.to(dev)[:, 1])
+            assert (again.double().cpu() - want).abs().max() < 2 * tol * want.abs().max()
+            if dtype == torch.bfloat16 and n * top <= 8:
+                # and every pair by the weight-streaming products that read on the device which expert is meant
+                y = ops.expert_pair_products(xd, w_gu.to(dtype).to(dev), w_d.to(dtype).to(dev), ids.to(dev))
+                own = torch.arange(n * top, dtype=torch.int32, device=dev).view(n, top)
+                third = ops.expert_combine(y, own, ids.to(dev), wts.to(dev), E, xd, shared.to(dtype).to(dev), sg.to(dev)[:, 1])
+                assert (third.double().cpu() - want).abs().max() < 2 * tol * want.abs().max()
 
 
 def test_norm_behind_a_branch_joined_with_the_next_norm():

@@ -76,6 +76,11 @@ struct NormArgs {
   const bf16_t* gain;  // [N]
   bf16_t* gained;
   float* sums_out;
+  // any variant: W is one of w_count matrices that lie w_stride elements apart, and which one is a number on the
+  // device, *w_select (clamped to the matrices there are), read when the kernel starts.  Null: W as it is.
+  const int32_t* w_select;
+  long long w_stride;
+  int w_count;
 };
 
 constexpr int kSumRows = 16;   // rows side by side in a piece of the sums of squares
@@ -116,6 +121,7 @@ gemm_stream_kernel(const bf16_t* __restrict__ A, int lda, const bf16_t* __restri
   const int step_lo = min(wave * steps_per_wave, steps_full);
   const int step_hi = min(step_lo + steps_per_wave, steps_full);
 
+  if (na.w_select != nullptr) W += (size_t)min(max(na.w_select[0], 0), na.w_count - 1) * (size_t)na.w_stride;
   // rows of W past N are clamped, rows of A past M read row 0: neither result is stored
   const bf16_t* wsrc[4 * NW];
 #pragma unroll
@@ -492,6 +498,28 @@ TL_EXPORT int tl_gemm_stream_glu(const void* A, int lda, const void* W, int ldw,
   NormArgs na = {};
   na.act = act;
   na.row_sums = row_sums; na.n_row_sums = n_row_sums; na.width = (float)K; na.eps = eps;
+  return run(A, lda, W, ldw, C, ldc, M, N, K, TL_BF16, waves, cols == 8 ? kGatedHalf : kGated, QkvArgs{}, na, stream);
+}
+
+// The plain and the gated product with a weight matrix chosen on the device: W points at the first of w_count
+// matrices that lie w_stride elements apart (a multiple of 8), and *w_select says which one this launch multiplies
+// with: an expert's weights, for a token whose expert only the device knows.
+TL_EXPORT int tl_gemm_stream_select(const void* A, int lda, const void* W, int ldw, void* C, int ldc, int M, int N, int K,
+                                    int out_dtype, int waves, const int32_t* w_select, long long w_stride, int w_count,
+                                    hipStream_t stream) {
+  TL_REQUIRE(w_select != nullptr && w_count > 0 && w_stride > 0 && w_stride % 8 == 0, "gemm_stream_select: bad choice of matrices");
+  NormArgs na = {};
+  na.w_select = w_select; na.w_stride = w_stride; na.w_count = w_count;
+  return run(A, lda, W, ldw, C, ldc, M, N, K, out_dtype, waves, kPlain, QkvArgs{}, na, stream);
+}
+
+TL_EXPORT int tl_gemm_stream_glu_select(const void* A, int lda, const void* W, int ldw, void* C, int ldc, int M, int N, int K,
+                                        int waves, int cols, const int32_t* w_select, long long w_stride, int w_count,
+                                        hipStream_t stream) {
+  TL_REQUIRE(cols == 8 || cols == 16, "gemm_stream_glu_select: cols must be 8 or 16");
+  TL_REQUIRE(w_select != nullptr && w_count > 0 && w_stride > 0 && w_stride % 8 == 0, "gemm_stream_glu_select: bad choice of matrices");
+  NormArgs na = {};
+  na.w_select = w_select; na.w_stride = w_stride; na.w_count = w_count;
   return run(A, lda, W, ldw, C, ldc, M, N, K, TL_BF16, waves, cols == 8 ? kGatedHalf : kGated, QkvArgs{}, na, stream);
 }
 

@@ -184,17 +184,14 @@ expert_down_rows_kernel(const T* __restrict__ mid, const T* __restrict__ w_d, co
 
 // The same two products for bfloat16 rows of up to NI * 512 elements, with the weights held in registers: a wave takes
 // one output, asks for its whole weight row (gate and up row) at once, 16 bytes a lane and round, and then walks the
-// expert's rows, at_once of them in LDS at a time.  The weights are read once however many rows the expert has, and every
-// load of a wave is in flight together.  GLU: w [E][2N][K], mid[r, n] = silu(gate) * up; else w [E][N][K], y[r, n] in 32-bit.
+// expert's rows.  The weights are read once however many rows the expert has, and every load of a wave is in flight
+// together.  GLU: w [E][2N][K], mid[r, n] = silu(gate) * up; else w [E][N][K], y[r, n] in 32-bit.
 // Each row's sum is taken in the order of the kernels above (a lane its rounds in ascending order, then the lanes).
 typedef __bf16 bf16x8_r __attribute__((ext_vector_type(8)));
-constexpr int kHeldRows = 4;
 template <int NI, bool GLU>
 __global__ void __launch_bounds__(kRowsThreads)
 expert_rows_held_kernel(const bf16_t* __restrict__ rows, const bf16_t* __restrict__ w, const int32_t* __restrict__ offsets,
-                        bf16_t* __restrict__ mid, float* __restrict__ y, int K, int N, int at_once) {
-  extern __shared__ __attribute__((aligned(16))) unsigned char lds_raw[];
-  bf16_t* x_l = reinterpret_cast<bf16_t*>(lds_raw);  // [at_once][K]
+                        bf16_t* __restrict__ mid, float* __restrict__ y, int K, int N) {
   const int e = blockIdx.x;
   const int lo = offsets[e], hi = offsets[e + 1];
   if (lo == hi) return;
@@ -211,44 +208,35 @@ expert_rows_held_kernel(const bf16_t* __restrict__ rows, const bf16_t* __restric
     gw[it] = *reinterpret_cast<const bf16x8_r*>(g_row + at);
     if (GLU) uw[it] = *reinterpret_cast<const bf16x8_r*>(u_row + at);
   }
-  for (int r0 = lo; r0 < hi; r0 += at_once) {
-    const int nr = min(at_once, hi - r0);
-    __syncthreads();
-    for (int i = threadIdx.x * 8; i < nr * K; i += kRowsThreads * 8)
-      *reinterpret_cast<bf16x8_r*>(x_l + i) = *reinterpret_cast<const bf16x8_r*>(rows + (size_t)r0 * K + i);
-    __syncthreads();
-    float ag[kHeldRows], au[kHeldRows];
+  // the expert's rows one after the other, each straight from memory (they are few and lie in the caches): the first
+  // row's pieces are asked for together with the weights, no LDS and no barrier
+  for (int r = lo; r < hi; ++r) {
+    const bf16_t* x_row = rows + (size_t)r * K;
+    bf16x8_r xv[NI];
 #pragma unroll
-    for (int r = 0; r < kHeldRows; ++r) ag[r] = au[r] = 0.f;
+    for (int it = 0; it < NI; ++it) {
+      const int d0 = (it * kWave + lane) * 8;
+      xv[it] = *reinterpret_cast<const bf16x8_r*>(x_row + (d0 < K ? d0 : 0));
+    }
+    float ag = 0.f, au = 0.f;
 #pragma unroll
     for (int it = 0; it < NI; ++it) {
       const int d0 = (it * kWave + lane) * 8;
       if (d0 < K) {
 #pragma unroll
-        for (int r = 0; r < kHeldRows; ++r) {
-          if (r < nr) {
-            const bf16x8_r xv = *reinterpret_cast<const bf16x8_r*>(x_l + r * K + d0);
-#pragma unroll
-            for (int i = 0; i < 8; ++i) {
-              const float xe = (float)xv[i];
-              ag[r] = fmaf((float)gw[it][i], xe, ag[r]);
-              if (GLU) au[r] = fmaf((float)uw[it][i], xe, au[r]);
-            }
-          }
+        for (int i = 0; i < 8; ++i) {
+          const float xe = (float)xv[it][i];
+          ag = fmaf((float)gw[it][i], xe, ag);
+          if (GLU) au = fmaf((float)uw[it][i], xe, au);
         }
       }
     }
-#pragma unroll
-    for (int r = 0; r < kHeldRows; ++r) {
-      if (r < nr) {
-        const float g = wave_sum(ag[r]);
-        if (GLU) {
-          const float u = wave_sum(au[r]);
-          if (live && lane == 0) mid[(size_t)(r0 + r) * N + n] = from_f32<bf16_t>(silu_r(g) * u);
-        } else {
-          if (live && lane == 0) y[(size_t)(r0 + r) * N + n] = g;
-        }
-      }
+    const float g = wave_sum(ag);
+    if (GLU) {
+      const float u = wave_sum(au);
+      if (live && lane == 0) mid[(size_t)r * N + n] = from_f32<bf16_t>(silu_r(g) * u);
+    } else {
+      if (live && lane == 0) y[(size_t)r * N + n] = g;
     }
   }
 }
@@ -332,13 +320,9 @@ static int launch_rows_held(const void* rows, const void* w, const int32_t* offs
     expert_rows_mfma_kernel<GLU><<<mgrid, kRowsThreads, 0, stream>>>((const bf16_t*)rows, (const bf16_t*)w, offsets, (bf16_t*)mid, y, K, N);
     return tl_check_launch("expert_rows_mfma");
   }
-  int at_once = 1;
-  while (at_once < kHeldRows && at_once < max_rows) at_once *= 2;
-  while (at_once > 1 && (size_t)at_once * K * 2 > 32 * 1024) at_once /= 2;
-  const size_t lds = (size_t)at_once * K * 2;
   const dim3 grid(n_experts, (N + kRowsThreads / kWave - 1) / (kRowsThreads / kWave));
   const int rounds = (K + kWave * 8 - 1) / (kWave * 8);
-#define TL_HELD(NI) expert_rows_held_kernel<NI, GLU><<<grid, kRowsThreads, lds, stream>>>((const bf16_t*)rows, (const bf16_t*)w, offsets, (bf16_t*)mid, y, K, N, at_once)
+#define TL_HELD(NI) expert_rows_held_kernel<NI, GLU><<<grid, kRowsThreads, 0, stream>>>((const bf16_t*)rows, (const bf16_t*)w, offsets, (bf16_t*)mid, y, K, N)
   if (rounds <= 1) TL_HELD(1);
   else if (rounds <= 2) TL_HELD(2);
   else if (rounds <= 4) TL_HELD(4);

@@ -59,6 +59,8 @@ _CORE_SIGNATURES = {
     "tl_softcap": [_P, _I64, _F, _P],
     "tl_gemm_f32": [_P, _I, _P, _I, _P, _I, _I, _I, _I, _P],
     "tl_gemm_stream": [_P, _I, _P, _I, _P, _I, _I, _I, _I, _I, _I, _P],
+    "tl_gemm_stream_select": [_P, _I, _P, _I, _P, _I, _I, _I, _I, _I, _I, _P, _I64, _I, _P],
+    "tl_gemm_stream_glu_select": [_P, _I, _P, _I, _P, _I, _I, _I, _I, _I, _I, _P, _I64, _I, _P],
     "tl_gemm_stream_glu": [_P, _I, _P, _I, _P, _I, _I, _I, _I, _I, _I, _P, _I, _F, _I, _P],
     "tl_gemm_stream_residual": [_P, _I, _P, _I, _P, _I, _P, _P, _P, _I, _P, _I, _I, _I, _I, _P],
     "tl_gemm_stream_qkv": [_P, _I, _P, _I, _P, _I, _I, _I, _I, _I, _I, _I, _P, _P, _P, _P, _I, _I, _P, _I, _F, _P],

@@ -125,6 +125,8 @@ from .routed_ops import (  # noqa: F401
     expert_down_rows,
     expert_gather,
     expert_glu_rows,
+    expert_pair_products,
+    PAIR_PRODUCTS_MOST,
     post_norm_add_norm,
     router_topk,
     weighted_pair,

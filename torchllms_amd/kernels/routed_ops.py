@@ -9,7 +9,7 @@ from typing import Optional, Tuple
 
 import torch
 
-from .base import KernelError, _gpu, _ptr, _stream, check, core, dtype_code
+from .base import F32, KernelError, _gpu, _ptr, _stream, check, core, dtype_code
 
 #: the most outputs a router may have (experts and experts that hand their input through together)
 ROUTER_MAX_OUTPUTS = 512
@@ -77,6 +77,44 @@ def expert_down_rows(mid: torch.Tensor, w_down: torch.Tensor, offsets: torch.Ten
     y = torch.empty((mid.shape[0], D), dtype=torch.float32, device=mid.device)
     check(core().tl_expert_down_rows(mid.data_ptr(), w_down.data_ptr(), offsets.data_ptr(), E, y.data_ptr(), D, F,
                                      mid.shape[0], dtype_code(mid.dtype), _stream()))
+    return y
+
+
+#: the most (token, choice) pairs of a bfloat16 step that ``expert_pair_products`` is meant for: every pair costs two
+#: launches, and each launch reads its expert's weights whoever else reads them too
+PAIR_PRODUCTS_MOST = 4
+
+
+def expert_pair_products(x: torch.Tensor, w_gate_up: torch.Tensor, w_down: torch.Tensor, ids: torch.Tensor) -> torch.Tensor:
+    """``y[t, j] = Wd[e] (silu(Wg[e] x[t]) * (Wu[e] x[t]))`` with ``e = ids[t, j]`` for the few pairs of a small decode
+    step, each pair by the weight-streaming products that dense layers use (bfloat16; the gate and up products are
+    rounded to bfloat16 before the activation, as theirs are), told on the device which expert's matrix to read.  A
+    pair whose ``e`` is no expert of the weights gets some expert's result, which nobody reads.  Returns float32
+    [n * top, D], the pairs in their own order."""
+    _gpu(x, w_gate_up, w_down, ids)
+    E = w_gate_up.shape[0] if w_gate_up.dim() == 3 else -1
+    _pairs(x, ids, E)
+    n, D = x.shape
+    if x.dtype != torch.bfloat16 or w_gate_up.dtype != x.dtype or w_down.dtype != x.dtype:
+        raise KernelError("expert_pair_products: bfloat16 rows and weights")
+    if w_gate_up.dim() != 3 or w_gate_up.shape[2] != D or w_gate_up.shape[1] % 2 or not w_gate_up.is_contiguous():
+        raise KernelError(f"expert_pair_products: gate and up weights must be contiguous [E, 2F, {D}]")
+    F = w_gate_up.shape[1] // 2
+    if tuple(w_down.shape) != (E, D, F) or not w_down.is_contiguous():
+        raise KernelError(f"expert_pair_products: down weights must be contiguous [{E}, {D}, {F}]")
+    if D % 8 or F % 8:
+        raise KernelError("expert_pair_products: widths must be multiples of 8")
+    top = ids.shape[1]
+    pairs = n * top
+    mid = torch.empty((pairs, F), dtype=x.dtype, device=x.device)
+    y = torch.empty((pairs, D), dtype=torch.float32, device=x.device)
+    lib, stream = core(), _stream()
+    for p in range(pairs):
+        which = ids.data_ptr() + 4 * p
+        check(lib.tl_gemm_stream_glu_select(x.data_ptr() + 2 * D * (p // top), D, w_gate_up.data_ptr(), D, mid.data_ptr() + 2 * F * p, F,
+                                            1, F, D, 0, 16, which, 2 * F * D, E, stream))
+        check(lib.tl_gemm_stream_select(mid.data_ptr() + 2 * F * p, F, w_down.data_ptr(), F, y.data_ptr() + 4 * D * p, D, 1, D, F,
+                                        F32, 0, which, D * F, E, stream))
     return y
 
 

@@ -84,7 +84,9 @@ class RoutedExperts(FeedForward):
     of them; each row's sums have an order of their own, so in 32-bit a token's result has the same bits in every
     step, and the launches are fixed by the step's shape (decode steps are replayed from graphs).  A bfloat16 step
     that brings prompts and has ``GROUPED_FROM`` pairs or more runs one matrix product per expert over its rows
-    instead; for that the host reads how many rows each expert got, once a layer."""
+    instead; for that the host reads how many rows each expert got, once a layer.  A bfloat16 step of at most
+    ``ops.PAIR_PRODUCTS_MOST`` pairs (one or two requests decoding) gathers nothing: every pair runs through the dense
+    layers' weight-streaming products, which read on the device which expert's matrix is meant."""
 
     graph_safe = True
     #: (token, choice) pairs of a bfloat16 step with prompts from which on the experts run as matrix products
@@ -98,6 +100,7 @@ class RoutedExperts(FeedForward):
             raise ValueError(f"routed: {top} choices among {num_experts} + {num_identity} outputs; sizes must not be negative")
         self.hidden_size, self.F, self.E, self.I, self.top, self.shared = hidden_size, expert_size, num_experts, num_identity, top, shared_size
         self.w_router = self.correction = self.w_gu = self.w_down = self.shared_w13 = self.shared_w2 = None
+        self._rows_in_order: Dict[int, torch.Tensor] = {}
 
     def param_specs(self) -> Dict[str, ParamSpec]:
         d, f, n = self.hidden_size, self.F, self.E + self.I
@@ -135,6 +138,13 @@ class RoutedExperts(FeedForward):
     def linear_weights(self):
         return [(self.w_router, "plain", torch.float32), (self.shared_w13, "glu"), self.shared_w2]
 
+    def _own_rows(self, n: int, device) -> torch.Tensor:
+        """int32 [n, top]: pair (t, j) lies in row t * top + j (results that were never put in the experts' order)."""
+        kept = self._rows_in_order.get(n)
+        if kept is None:
+            kept = self._rows_in_order[n] = torch.arange(n * self.top, dtype=torch.int32, device=device).view(n, self.top).contiguous()
+        return kept
+
     def forward(self, x, ctx):
         x = ops.resolved(x)
         n_out = self.E + self.I
@@ -144,6 +154,11 @@ class RoutedExperts(FeedForward):
         if self.shared:
             shared = ops.linear(ops.linear_glu(x, self.shared_w13), self.shared_w2)
             gate = z[:, n_out]
+        pairs = x.shape[0] * self.top
+        if x.dtype == torch.bfloat16 and pairs <= ops.PAIR_PRODUCTS_MOST and self.hidden_size % 8 == 0 and self.F % 8 == 0:
+            # a decode step of one or two requests: every pair by the dense layers' weight-streaming products
+            y = ops.expert_pair_products(x, self.w_gu, self.w_down, ids)
+            return ops.expert_combine(y, self._own_rows(x.shape[0], x.device), ids, weights, self.E, x, shared, gate)
         rows, pos, offsets = ops.expert_gather(x, ids, n_out)
         if x.dtype == torch.float32 or ctx.host.max_q_len <= 1 or x.shape[0] * self.top < self.GROUPED_FROM:
             y = ops.expert_down_rows(ops.expert_glu_rows(rows, self.w_gu, offsets), self.w_down, offsets)
