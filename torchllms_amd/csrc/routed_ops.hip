@@ -382,18 +382,20 @@ __global__ void __launch_bounds__(256)
 expert_combine_kernel(const YT* __restrict__ y, const int32_t* __restrict__ pos, const int32_t* __restrict__ ids,
                       const float* __restrict__ weights, int top, int n_experts, const T* __restrict__ x,
                       const T* __restrict__ shared, const float* __restrict__ sg, int sg_stride, T* __restrict__ out, int D) {
+  // a block a token and 256 columns: a token's few columns are spread over many blocks, so that a step of few tokens is
+  // not one block's walk along the row
   const int t = blockIdx.x;
+  const int d = blockIdx.y * blockDim.x + threadIdx.x;
+  if (d >= D) return;
   const float share = shared ? sigmoid_r(sg[(size_t)t * sg_stride]) : 0.f;
-  for (int d = threadIdx.x; d < D; d += blockDim.x) {
-    float total = 0.f;
-    for (int j = 0; j < top; ++j) {
-      const int e = ids[(size_t)t * top + j];
-      const float wj = weights[(size_t)t * top + j];
-      total += wj * (e < n_experts ? to_f32(y[(size_t)pos[(size_t)t * top + j] * D + d]) : to_f32(x[(size_t)t * D + d]));
-    }
-    if (shared) total += share * to_f32(shared[(size_t)t * D + d]);
-    out[(size_t)t * D + d] = from_f32<T>(total);
+  float total = 0.f;
+  for (int j = 0; j < top; ++j) {
+    const int e = ids[(size_t)t * top + j];
+    const float wj = weights[(size_t)t * top + j];
+    total += wj * (e < n_experts ? to_f32(y[(size_t)pos[(size_t)t * top + j] * D + d]) : to_f32(x[(size_t)t * D + d]));
   }
+  if (shared) total += share * to_f32(shared[(size_t)t * D + d]);
+  out[(size_t)t * D + d] = from_f32<T>(total);
 }
 
 // ----------------------------------------------------------------------------- dense feed-forward with biases
@@ -610,11 +612,12 @@ TL_EXPORT int tl_expert_gather(const void* x, const int32_t* ids, int n, int top
 TL_EXPORT int tl_expert_combine(const void* y, int y_f32, const int32_t* pos, const int32_t* ids, const float* weights, int top,
                                 int n_experts, const void* x, const void* shared, const float* sg, int sg_stride, void* out, int n,
                                 int D, int dtype, hipStream_t stream) {
-  TL_REQUIRE(n >= 0 && top > 0 && n_experts >= 0 && D > 0, "expert_combine: bad sizes");
+  TL_REQUIRE(n >= 0 && n <= 0x7fffffff && top > 0 && n_experts >= 0 && D > 0 && (D + 255) / 256 <= 65535, "expert_combine: bad sizes");
   TL_REQUIRE(shared == nullptr || sg != nullptr, "expert_combine: a shared expert without its gate");
   if (n == 0) return TL_OK;
+  const dim3 cgrid(n, (D + 255) / 256);
 #define TL_COMBINE(T, YT)                                                                                                   \
-  expert_combine_kernel<T, YT><<<n, 256, 0, stream>>>((const YT*)y, pos, ids, weights, top, n_experts, (const T*)x, (const T*)shared, \
+  expert_combine_kernel<T, YT><<<cgrid, 256, 0, stream>>>((const YT*)y, pos, ids, weights, top, n_experts, (const T*)x, (const T*)shared, \
                                                       sg, sg_stride, (T*)out, D)
   if (dtype == TL_F32) TL_COMBINE(float, float);
   else if (dtype == TL_BF16 && y_f32) TL_COMBINE(bf16_t, float);
