@@ -168,7 +168,7 @@ class RoutedExperts(FeedForward):
         for e in range(self.E):
             lo, hi = bounds[e], bounds[e + 1]
             if hi > lo:
-                parts.append(ops.linear(ops.linear_glu(rows[lo:hi], self.w_gu[e]), self.w_down[e]))
+                parts.append(ops.linear(ops.linear_glu(rows[lo:hi], self.w_gu[e]), self.w_down[e], out_dtype=torch.float32))
         # (the rows of experts that hand their input through lie behind all others and are never read)
-        y = torch.cat(parts) if parts else rows
+        y = torch.cat(parts) if parts else rows  # (32-bit results: the weighted sum rounds once)
         return ops.expert_combine(y, pos, ids, weights, self.E, x, shared, gate)
