@@ -616,6 +616,50 @@ def test_trace_replay_program(tmp_path):
             assert distance(row, truth[rid][pos], scale) < FP32_TOL
 
 
+# ----------------------------------------------------------------------------- sizes that no vector load divides
+ODD = {
+    "width_100": models.model(301, 100, 1.5, 1e-6, [
+        models.layer("parallel", models.pair(models.left(3, 1, 20, 6, 0.2), models.right(3, 3, 12, 20, 3, 3, 5), 0.6, 0.5),
+                     models.moe(36, 5, 2, identity=1, shared=20)),
+        models.layer("mlstm", models.mlstm(5, 12, 20, 15.0), models.dense(52)),
+        models.layer("mlstm", models.mlstm(2, 30, 50, 15.0), models.moe(28, 3, 3, identity=4)),
+    ]),
+    "width_36": models.model(97, 36, 3.0, 1e-6, [
+        models.layer("mlstm", models.mlstm(1, 10, 6, 4.0), models.moe(12, 9, 4, identity=4, shared=4)),
+        models.layer("parallel", models.pair(models.left(9, 3, 8, 8, 0.35, base=1e6), models.right(4, 1, 10, 14, 4, 2, 2), 0.6, 0.5), None),
+    ]),
+}
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+@pytest.mark.parametrize("name", sorted(ODD))
+def test_widths_that_are_no_multiple_of_eight(tmp_path, name, dtype):
+    """Rows of 100 and 36 channels, experts of 36, 28 and 12, heads of 20, 12, 10 and 8, more experts that hand their
+    input through than experts: the kernels' forms for rows that no 16-byte load divides, a prompt whole and then a
+    prompt with its last 50 tokens one by one."""
+    from torchllms_amd.engine import Engine, StepEntry
+
+    cfg_dict = ODD[name]
+    folder = folder_for(dtype, tmp_path / name, cfg_dict, seed=3)
+    tokens = random_tokens(150, cfg_dict["vocab"], 4)
+    truth, scale = truth_of(*models.read_folder(folder), {"r": tokens})
+    engine = Engine.from_folder(folder, dtype=dtype, page_size=16, num_pages=40, max_seqs=2)
+    engine.admit("a")
+    whole = engine.step([StepEntry("a", tokens, list(range(150)))]).cpu()
+    engine.admit("b")
+    rows = [engine.step([StepEntry("b", tokens[:100], list(range(100)))]).cpu()]
+    rows += [engine.step([StepEntry("b", [t], [0])]).cpu() for t in tokens[100:]]
+    cut = torch.cat(rows)
+    for got in (whole, cut):
+        dists = [distance(got[i], truth["r"][i], scale) for i in range(150)]
+        if dtype == "float32":
+            assert max(dists) < FP32_TOL
+        else:
+            assert_within_rounding(dists, 1.5 * BF16_TOL, name)
+    if dtype == "float32":
+        assert torch.equal(whole, cut)
+
+
 # ----------------------------------------------------------------------------- random configurations
 def random_config(seed: int) -> dict:
     """A Kepevik configuration drawn from a seed: every size, constant and the order of layers."""
