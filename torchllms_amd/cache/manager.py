@@ -48,6 +48,8 @@ class CacheGroupSpec:
     dtype: Optional[str] = None  # "float32" / "bfloat16"; None: the manager's default
     v_head_dim: int = 0  # head size of the values; 0: that of the keys
     values_in_keys: bool = False  # a token's value is the first channels of its key row: no value pages
+    keep_first: int = 0  # with a window: the first positions of a request stay visible, their pages stay held
+    v_heads: int = 0  # heads of the value pages; 0: as many as the key pages have
 
     @property
     def value_dim(self) -> int:
@@ -56,7 +58,11 @@ class CacheGroupSpec:
     @property
     def elements_per_token(self) -> int:
         """Cached elements of one token in one layer of the group."""
-        return self.num_kv_heads * (self.head_dim + (0 if self.values_in_keys else self.value_dim))
+        return self.num_kv_heads * self.head_dim + (0 if self.values_in_keys else self.value_heads * self.value_dim)
+
+    @property
+    def value_heads(self) -> int:
+        return self.v_heads or self.num_kv_heads
 
 
 @dataclass(frozen=True)
@@ -81,7 +87,9 @@ def group_layers(needs: Sequence[Tuple[Hashable, object]]) -> Tuple[List[CacheGr
         if hasattr(need, "num_kv_heads"):
             v_dim = int(getattr(need, "v_head_dim", None) or 0)
             form = (need.num_kv_heads, need.head_dim, need.window, int(getattr(need, "page_size", None) or 0),
-                    getattr(need, "dtype", None), 0 if v_dim == need.head_dim else v_dim, bool(getattr(need, "values_in_keys", False)))
+                    getattr(need, "dtype", None), 0 if v_dim == need.head_dim else v_dim, bool(getattr(need, "values_in_keys", False)),
+                    int(getattr(need, "keep_first", 0) or 0) if need.window > 0 else 0,
+                    0 if int(getattr(need, "num_v_heads", None) or 0) == need.num_kv_heads else int(getattr(need, "num_v_heads", None) or 0))
             kv.setdefault(form, []).append(run_id)
         elif hasattr(need, "shape"):
             st.setdefault((tuple(need.shape), need.dtype), []).append(run_id)
@@ -89,8 +97,8 @@ def group_layers(needs: Sequence[Tuple[Hashable, object]]) -> Tuple[List[CacheGr
             raise TypeError(f"cache entry {run_id}: unknown cache need {need!r}")
     groups = [
         CacheGroupSpec(name=f"kv{i}", run_ids=tuple(runs), num_kv_heads=h, head_dim=d, window=w, page_size=p, dtype=t,
-                       v_head_dim=vd, values_in_keys=vk)
-        for i, ((h, d, w, p, t, vd, vk), runs) in enumerate(kv.items())
+                       v_head_dim=vd, values_in_keys=vk, keep_first=kf, v_heads=vh)
+        for i, ((h, d, w, p, t, vd, vk, kf, vh), runs) in enumerate(kv.items())
     ]
     states = [
         StateSlotSpec(name=f"state{i}", run_ids=tuple(runs), shape=shape, dtype=dtype)
@@ -227,8 +235,8 @@ class CacheManager:
                 shape = (len(g.run_ids), pool.num_pages, g.num_kv_heads, self.page_sizes[gi])
                 self.k_pages.append(torch.zeros(shape + (g.head_dim,), dtype=self.dtypes[gi], device=device))
                 # (values that live inside the key rows: the mixer's value pages are its key pages)
-                self.v_pages.append(self.k_pages[-1] if g.values_in_keys else
-                                    torch.zeros(shape + (g.value_dim,), dtype=self.dtypes[gi], device=device))
+                v_shape = (len(g.run_ids), pool.num_pages, g.value_heads, self.page_sizes[gi], g.value_dim)
+                self.v_pages.append(self.k_pages[-1] if g.values_in_keys else torch.zeros(v_shape, dtype=self.dtypes[gi], device=device))
             for s in self.states:
                 shape = (len(s.run_ids), max_seqs, *s.shape)
                 self.state_tensors.append(torch.zeros(shape, dtype=getattr(torch, s.dtype), device=device))
@@ -327,6 +335,12 @@ class CacheManager:
         lo = first_query_pos - w + 1
         return max(lo, 0) // self.page_sizes[group]
 
+    def kept_blocks(self, group: int) -> int:
+        """The first blocks of a request that a window of ``group`` never passes: those that hold the first positions
+        that stay visible (``keep_first``)."""
+        g = self.groups[group]
+        return -(-g.keep_first // self.page_sizes[group]) if g.window > 0 and g.keep_first > 0 else 0
+
     def pages_short(self, rid: Hashable, n_new: int) -> Dict[int, int]:
         """Per group, how many pages are missing to take ``n_new`` more tokens (0 if it fits)."""
         e = self.entry(rid)
@@ -386,10 +400,11 @@ class CacheManager:
         for gi, pool in enumerate(self.pools):
             first = min(self._first_needed_block(gi, e.num_tokens), len(e.block_tables[gi]))
             bt = e.block_tables[gi]
-            passed = [bt[b] for b in range(e.first_live_block[gi], first) if bt[b] >= 0]
+            behind = range(max(e.first_live_block[gi], self.kept_blocks(gi)), first)  # (the kept first blocks stay)
+            passed = [bt[b] for b in behind if bt[b] >= 0]
             if passed:
                 pool.give_back(passed)
-                for b in range(e.first_live_block[gi], first):
+                for b in behind:
                     bt[b] = -1
                 e.table_arrays[gi] = None
             e.first_live_block[gi] = max(e.first_live_block[gi], first)
@@ -403,7 +418,7 @@ class CacheManager:
         for gi, pool in enumerate(self.pools):
             bt = e.block_tables[gi]
             keep = self.blocks_for(num_tokens, gi)
-            if keep < e.first_live_block[gi]:
+            if keep < e.first_live_block[gi] and e.first_live_block[gi] > self.kept_blocks(gi):
                 raise ValueError("cannot truncate into pages a window has already released")
             tail = [p for p in bt[keep:] if p >= 0]
             pool.give_back(tail)
@@ -467,7 +482,7 @@ class CacheManager:
         page_size = self.page_sizes[gi]
         n = e.num_tokens
         k = torch.zeros((n, g.num_kv_heads, g.head_dim), dtype=self.dtypes[gi], device=self.device)
-        v = torch.zeros((n, g.num_kv_heads, g.head_dim if g.values_in_keys else g.value_dim), dtype=self.dtypes[gi], device=self.device)
+        v = torch.zeros((n, g.value_heads, g.head_dim if g.values_in_keys else g.value_dim), dtype=self.dtypes[gi], device=self.device)
         for b, page in enumerate(e.block_tables[gi]):
             lo = b * page_size
             hi = min(lo + page_size, n)
@@ -492,12 +507,13 @@ class CacheManager:
                     raise AssertionError(f"{rid!r}: {len(bt)} blocks for {e.num_tokens} tokens")
                 if len(bt) > need:
                     raise AssertionError(f"{rid!r}: holds {len(bt)} blocks, needs at most {need}")
+                kept = self.kept_blocks(gi)
                 for b, p in enumerate(bt):
                     if p < 0:
-                        if b >= e.first_live_block[gi]:
+                        if b >= e.first_live_block[gi] or b < kept:
                             raise AssertionError(f"{rid!r}: live block {b} has no page")
                         continue
-                    if b < e.first_live_block[gi]:
+                    if kept <= b < e.first_live_block[gi]:
                         raise AssertionError(f"{rid!r}: block {b} is behind the window but still holds page {p}")
                     held[p] = held.get(p, 0) + 1
             free = pool._free

@@ -19,6 +19,7 @@ from .spec import ModelSpec
 from .taluvik import ARCHITECTURE as TALUVIK, TaluvikConfig, taluvik_model_spec
 from .vobolorn import ARCHITECTURE as VOBOLORN, VobolornConfig, vobolorn_model_spec
 from .kepevik import ARCHITECTURE as KEPEVIK, KepevikConfig, kepevik_model_spec, kepevik_sizes_from_tensors
+from .nosuzen import ARCHITECTURE as NOSUZEN, NosuzenConfig, nosuzen_model_spec, nosuzen_sizes_from_tensors
 
 
 @dataclass(frozen=True)
@@ -223,5 +224,29 @@ register_architecture(
         stop_token_ids=_kepevik_stop_ids,
         config_type=KepevikConfig,
         sizes_from_tensors=kepevik_sizes_from_tensors,
+    )
+)
+
+
+def _nosuzen_rules(cfg: NosuzenConfig):
+    from ..weights.names import nosuzen_name_rules
+
+    return nosuzen_name_rules(cfg)
+
+
+def _nosuzen_stop_ids(cfg: NosuzenConfig):
+    eos = cfg.eos_token_id
+    return [] if eos is None else (list(eos) if isinstance(eos, (list, tuple)) else [eos])
+
+
+register_architecture(
+    ArchSpec(
+        name=NOSUZEN,
+        config_from_dict=NosuzenConfig.from_dict,
+        model_spec=nosuzen_model_spec,
+        weight_rules=_nosuzen_rules,
+        stop_token_ids=_nosuzen_stop_ids,
+        config_type=NosuzenConfig,
+        sizes_from_tensors=nosuzen_sizes_from_tensors,
     )
 )

@@ -6,7 +6,10 @@
 // the bfloat16 path for sizes the MFMA kernels refuse.  Beyond the plain form it takes: values of
 // another head size than the keys (v_dim), a cap on the scores (s <- cap * tanh(s / cap)), chunks
 // (a query sees only keys of its own chunk of `chunk` positions, counted from position 0) and a sink
-// per query head (one more term exp(sink) in the softmax's denominator, without a value).
+// per query head (one more term exp(sink) in the softmax's denominator, without a value), first keys that stay
+// visible behind a window (keep_first: a query also sees the positions below it that lie before its window), and
+// values with fewer heads than the keys (key head g reads value head g mod n_v_heads: several score maps over
+// the same values).
 #include <limits.h>
 
 #include "common.h"
@@ -52,7 +55,9 @@ struct Query {
   const T* v_pages;
   const int32_t* bt;        // the request's block table
   int n_kv_heads, g, head_dim, v_dim, v_pitch, page_size;  // v_pitch: elements between two value rows
+  int n_v_heads, gv;        // heads of the value pages, and the one this query reads
   int lo, p;                // the keys it sees: positions lo .. p
+  int keep;                 // and positions 0 .. keep - 1 before them (kept first keys; keep <= lo)
   float scale, softcap;
 };
 
@@ -86,11 +91,12 @@ __device__ __forceinline__ void block_partial(const Query<T>& a, int j0, int lan
   const int j = j0 + lane;
   const bool valid = j >= a.lo && j <= a.p;
   float s = -INFINITY;
-  long long row_at = 0;  // index of this lane's key (and value) row in the pages
+  long long row_at = 0;  // index of this lane's value row in the pages
   if (valid) {
     const int page = a.bt[j / a.page_size];
-    row_at = (long long)(((size_t)page * a.n_kv_heads + a.g) * a.page_size + (size_t)(j % a.page_size));
-    const T* kr = a.k_pages + row_at * a.head_dim;
+    const long long key_at = (long long)(((size_t)page * a.n_kv_heads + a.g) * a.page_size + (size_t)(j % a.page_size));
+    row_at = (long long)(((size_t)page * a.n_v_heads + a.gv) * a.page_size + (size_t)(j % a.page_size));
+    const T* kr = a.k_pages + key_at * a.head_dim;
     float dot = 0.f;
     if (VEC) {
       // eight pieces of the row are asked for before the first is multiplied (a piece past the row's end is
@@ -172,7 +178,8 @@ __device__ __forceinline__ Query<T> make_query(const float* qs, const T* k_pages
                                                const int32_t* token_seq, const int32_t* positions,
                                                const int32_t* block_table, int bt_stride, int t, int h, int n_q_heads,
                                                int n_kv_heads, int head_dim, int page_size, int window, float scale,
-                                               float softcap, int chunk, int v_dim, int v_pitch) {
+                                               float softcap, int chunk, int v_dim, int v_pitch, int keep_first,
+                                               int n_v_heads) {
   Query<T> a;
   a.qs = qs; a.k_pages = k_pages; a.v_pages = v_pages;
   a.bt = block_table + (size_t)token_seq[t] * bt_stride;
@@ -180,8 +187,31 @@ __device__ __forceinline__ Query<T> make_query(const float* qs, const T* k_pages
   a.page_size = page_size;
   a.p = positions[t];
   a.lo = first_key(a.p, window, chunk);
+  a.keep = min(keep_first, a.lo);
+  a.n_v_heads = n_v_heads; a.gv = a.g % n_v_heads;
   a.scale = scale; a.softcap = softcap;
   return a;
+}
+
+// All blocks of a query, by one wave: first the kept first keys (positions 0 .. keep - 1, as blocks of their own,
+// also where the last of them shares its 64 positions with the window's first), then positions lo .. p.
+template <typename T, bool VEC>
+__device__ __forceinline__ void walk_alone(const Query<T>& a, int lane, float& m, float& l, float (&acc)[kChanPerLane]) {
+  if (a.keep > 0) {
+    Query<T> first = a;
+    first.lo = 0;
+    first.p = a.keep - 1;
+    for (int j0 = 0; j0 < a.keep; j0 += kWave) {
+      float m_b, l_b, o_b[kChanPerLane];
+      block_partial<T, VEC>(first, j0, lane, m_b, l_b, o_b);
+      merge_block(m, l, acc, m_b, l_b, o_b);
+    }
+  }
+  for (int j0 = a.lo - a.lo % kWave; j0 <= a.p; j0 += kWave) {
+    float m_b, l_b, o_b[kChanPerLane];
+    block_partial<T, VEC>(a, j0, lane, m_b, l_b, o_b);
+    merge_block(m, l, acc, m_b, l_b, o_b);
+  }
 }
 
 // One wave per (token, query head) walks all blocks of 64 keys in ascending order.  It works alone:
@@ -193,7 +223,7 @@ attention_generic_kernel(const T* __restrict__ q, int q_stride, T* __restrict__ 
                          const int32_t* __restrict__ token_seq, const int32_t* __restrict__ positions,
                          const int32_t* __restrict__ block_table, int bt_stride, int n_q_heads,
                          int n_kv_heads, int head_dim, int page_size, int window, float scale, float softcap,
-                         int chunk, const float* __restrict__ sinks, int v_dim, int v_pitch) {
+                         int chunk, const float* __restrict__ sinks, int v_dim, int v_pitch, int keep_first, int n_v_heads) {
   __shared__ float q_lds[kWavesPerBlock][kMaxKeyDim];
   const int t = blockIdx.x;
   const int wave = threadIdx.x / kWave;
@@ -205,16 +235,12 @@ attention_generic_kernel(const T* __restrict__ q, int q_stride, T* __restrict__ 
   for (int d = lane; d < head_dim; d += kWave) q_lds[wave][d] = to_f32(qv[d]);
   __syncthreads();
   const Query<T> a = make_query<T>(q_lds[wave], k_pages, v_pages, token_seq, positions, block_table, bt_stride, t, h,
-                                   n_q_heads, n_kv_heads, head_dim, page_size, window, scale, softcap, chunk, v_dim, v_pitch);
+                                   n_q_heads, n_kv_heads, head_dim, page_size, window, scale, softcap, chunk, v_dim, v_pitch, keep_first, n_v_heads);
   float acc[kChanPerLane];
 #pragma unroll
   for (int c = 0; c < kChanPerLane; ++c) acc[c] = 0.f;
   float m = -INFINITY, l = 0.f;
-  for (int j0 = a.lo - a.lo % kWave; j0 <= a.p; j0 += kWave) {
-    float m_b, l_b, o_b[kChanPerLane];
-    block_partial<T, VEC>(a, j0, lane, m_b, l_b, o_b);
-    merge_block(m, l, acc, m_b, l_b, o_b);
-  }
+  walk_alone<T, VEC>(a, lane, m, l, acc);
   if (active) {
     T* o = out + (size_t)t * out_stride + (size_t)h * v_dim;
     const float inv_l = 1.0f / with_sink(l, m, sinks, h);
@@ -303,7 +329,8 @@ attention_tile_kernel(const T* __restrict__ q, int q_stride, T* __restrict__ out
                       const int32_t* __restrict__ token_seq, const int32_t* __restrict__ positions,
                       const int32_t* __restrict__ block_table, int bt_stride, int n_tokens, int n_q_heads,
                       int n_kv_heads, int head_dim, int page_size, int window, float scale, int heads_per_block,
-                      float softcap, int chunk, const float* __restrict__ sinks, int v_dim, int v_pitch) {
+                      float softcap, int chunk, const float* __restrict__ sinks, int v_dim, int v_pitch, int keep_first,
+                      int n_v_heads) {
   extern __shared__ __attribute__((aligned(16))) float tile_lds[];
   const int pitch = head_dim + kTilePad, pitch_v = v_dim + kTilePad;
   float* q_lds = tile_lds;                          // [kTileWaves][head_dim]
@@ -323,16 +350,17 @@ attention_tile_kernel(const T* __restrict__ q, int q_stride, T* __restrict__ out
   for (int d = lane; d < head_dim; d += kWave) q_lds[wave * head_dim + d] = to_f32(qv[d]);
   const Query<T> a = make_query<T>(q_lds + wave * head_dim, k_pages, v_pages, token_seq, positions, block_table,
                                    bt_stride, t, h, n_q_heads, n_kv_heads, head_dim, page_size, window, scale, softcap,
-                                   chunk, v_dim, v_pitch);
+                                   chunk, v_dim, v_pitch, keep_first, n_v_heads);
   // what the whole block sees: the same for every thread, from the tokens' own entries
   const int last = min(t0 + QT, n_tokens) - 1;
   const int seq0 = token_seq[t0];
   bool together = true;
-  int blk_lo = INT_MAX, blk_hi = -1, key_lo = INT_MAX;
+  int blk_lo = INT_MAX, blk_hi = -1, key_lo = INT_MAX, keep_hi = 0;
   for (int i = t0; i <= last; ++i) {
     together = together && token_seq[i] == seq0;
     const int pi = positions[i];
     const int li = first_key(pi, window, chunk);
+    keep_hi = max(keep_hi, min(keep_first, li));
     blk_lo = min(blk_lo, li - li % kWave);
     key_lo = min(key_lo, li);
     blk_hi = max(blk_hi, pi);
@@ -340,34 +368,37 @@ attention_tile_kernel(const T* __restrict__ q, int q_stride, T* __restrict__ out
   __syncthreads();  // the queries are in LDS
   // the wave's own bounds, as scalars (they are the same in all its lanes)
   const int lo_u = __builtin_amdgcn_readfirstlane(a.lo), p_u = __builtin_amdgcn_readfirstlane(a.p);
+  const int keep_u = __builtin_amdgcn_readfirstlane(a.keep);
   float acc[kChanPerLane];
 #pragma unroll
   for (int c = 0; c < kChanPerLane; ++c) acc[c] = 0.f;
   float m = -INFINITY, l = 0.f;
   if (!together) {
-    for (int j0 = a.lo - a.lo % kWave; j0 <= a.p; j0 += kWave) {
-      float m_b, l_b, o_b[kChanPerLane];
-      block_partial<T, VEC>(a, j0, lane, m_b, l_b, o_b);
-      merge_block(m, l, acc, m_b, l_b, o_b);
-    }
+    walk_alone<T, VEC>(a, lane, m, l, acc);
   } else {
     const int g = (blockIdx.y * HB) / (n_q_heads / n_kv_heads);  // the kv head of all the block's heads
+    const int gv = g % n_v_heads;
     const int32_t* bt = block_table + (size_t)seq0 * bt_stride;
     // pieces of a key row and of a value row: four elements, or one
     const int per_k = VEC ? head_dim / 4 : head_dim, per_v = VEC ? v_dim / 4 : v_dim;
     const int per_row = per_k + per_v;
-    for (int j0 = blk_lo; j0 <= blk_hi; j0 += kWave) {
-      if (j0 > blk_lo) __syncthreads();  // everybody has finished with the tiles of the block before
+    bool first_pass = true;
+    // one block of 64 keys for everybody: the keys load_lo .. load_hi of it into LDS, then every wave whose range
+    // lo_w .. p_w touches the block takes it in
+    auto pass = [&](int j0, int load_lo, int load_hi, int lo_w, int p_w) {
+      if (!first_pass) __syncthreads();  // everybody has finished with the tiles of the block before
+      first_pass = false;
       for (int idx = threadIdx.x; idx < kWave * per_row; idx += kTileWaves * kWave) {
         const int r = idx / per_row, piece_kv = idx % per_row;
         const int j = j0 + r;
-        if (j < key_lo || j > blk_hi) continue;  // nobody in the block sees this key
+        if (j < load_lo || j > load_hi) continue;  // nobody in the block sees this key
         const int page = bt[j / page_size];
         if (page < 0) continue;  // a page that a window gave back: no token of the step sees its keys
         const size_t row_at = ((size_t)page * n_kv_heads + g) * page_size + (size_t)(j % page_size);
+        const size_t val_at = ((size_t)page * n_v_heads + gv) * page_size + (size_t)(j % page_size);
         const bool is_k = piece_kv < per_k;
         const int piece = is_k ? piece_kv : piece_kv - per_k;
-        const T* src = is_k ? k_pages + row_at * head_dim : v_pages + row_at * v_pitch;
+        const T* src = is_k ? k_pages + row_at * head_dim : v_pages + val_at * v_pitch;
         float* dst = is_k ? k_t + r * pitch : v_t + r * pitch_v;
         if (VEC) {
           float e[4];
@@ -378,13 +409,15 @@ attention_tile_kernel(const T* __restrict__ q, int q_stride, T* __restrict__ out
         }
       }
       __syncthreads();
-      if (j0 >= lo_u - lo_u % kWave && j0 <= p_u) {  // (uniform per wave)
+      if (p_w >= lo_w && j0 >= lo_w - lo_w % kWave && j0 <= p_w) {  // (uniform per wave)
         float m_b, l_b, o_b[kChanPerLane];
-        block_partial_lds<VEC, CH>(a.qs, k_t, v_t, pitch, pitch_v, head_dim, v_dim, lo_u, p_u, scale, softcap, j0, lane,
+        block_partial_lds<VEC, CH>(a.qs, k_t, v_t, pitch, pitch_v, head_dim, v_dim, lo_w, p_w, scale, softcap, j0, lane,
                                    m_b, l_b, o_b);
         merge_block(m, l, acc, m_b, l_b, o_b);
       }
-    }
+    };
+    for (int j0 = 0; j0 < keep_hi; j0 += kWave) pass(j0, 0, keep_hi - 1, 0, keep_u - 1);  // the kept first keys
+    for (int j0 = blk_lo; j0 <= blk_hi; j0 += kWave) pass(j0, key_lo, blk_hi, lo_u, p_u);
   }
   if (active) {
     T* o = out + (size_t)t * out_stride + (size_t)h * v_dim;
@@ -409,7 +442,8 @@ attention_blocks_kernel(const T* __restrict__ q, int q_stride, const T* __restri
                         const T* __restrict__ v_pages, const int32_t* __restrict__ token_seq,
                         const int32_t* __restrict__ positions, const int32_t* __restrict__ block_table, int bt_stride,
                         int n_q_heads, int n_kv_heads, int head_dim, int page_size, int window, float scale,
-                        float* __restrict__ partials, int max_blocks, float softcap, int chunk, int v_dim, int v_pitch) {
+                        float* __restrict__ partials, int max_blocks, float softcap, int chunk, int v_dim, int v_pitch,
+                        int keep_first, int n_v_heads) {
   __shared__ float q_lds[kWavesPerBlock][kMaxKeyDim];
   const int t = blockIdx.x;
   const int r = blockIdx.z;
@@ -422,11 +456,21 @@ attention_blocks_kernel(const T* __restrict__ q, int q_stride, const T* __restri
   for (int d = lane; d < head_dim; d += kWave) q_lds[wave][d] = to_f32(qv[d]);
   __syncthreads();
   const Query<T> a = make_query<T>(q_lds[wave], k_pages, v_pages, token_seq, positions, block_table, bt_stride, t, h,
-                                   n_q_heads, n_kv_heads, head_dim, page_size, window, scale, softcap, chunk, v_dim, v_pitch);
-  const int j0 = a.lo - a.lo % kWave + r * kWave;
-  if (j0 > a.p || !active) return;  // (uniform per wave)
+                                   n_q_heads, n_kv_heads, head_dim, page_size, window, scale, softcap, chunk, v_dim, v_pitch, keep_first, n_v_heads);
+  // the blocks of the kept first keys come first, then those of positions lo .. p
+  const int kept_blocks = (a.keep + kWave - 1) / kWave;
+  Query<T> b = a;
+  int j0;
+  if (r < kept_blocks) {
+    b.lo = 0;
+    b.p = a.keep - 1;
+    j0 = r * kWave;
+  } else {
+    j0 = a.lo - a.lo % kWave + (r - kept_blocks) * kWave;
+  }
+  if (j0 > b.p || !active) return;  // (uniform per wave)
   float m_b, l_b, o_b[kChanPerLane];
-  block_partial<T, VEC>(a, j0, lane, m_b, l_b, o_b);
+  block_partial<T, VEC>(b, j0, lane, m_b, l_b, o_b);
   float* dst = partials + (((size_t)t * n_q_heads + h) * max_blocks + r) * (v_dim + kPartialExtra);
 #pragma unroll
   for (int c = 0; c < kChanPerLane; ++c) {
@@ -443,7 +487,7 @@ template <typename T>
 __global__ void __launch_bounds__(kWavesPerBlock* kWave)
 attention_join_kernel(T* __restrict__ out, int out_stride, const int32_t* __restrict__ positions, int n_q_heads,
                       int head_dim, int window, const float* __restrict__ partials, int max_blocks, int chunk,
-                      const float* __restrict__ sinks) {  // (head_dim: the values' head size)
+                      const float* __restrict__ sinks, int keep_first) {  // (head_dim: the values' head size)
   const int t = blockIdx.x;
   const int wave = threadIdx.x / kWave;
   const int lane = threadIdx.x % kWave;
@@ -451,7 +495,7 @@ attention_join_kernel(T* __restrict__ out, int out_stride, const int32_t* __rest
   if (h >= n_q_heads) return;
   const int p = positions[t];
   const int lo = first_key(p, window, chunk);
-  const int n_blocks = (p - (lo - lo % kWave)) / kWave + 1;
+  const int n_blocks = (min(keep_first, lo) + kWave - 1) / kWave + (p - (lo - lo % kWave)) / kWave + 1;
   const int stride = head_dim + kPartialExtra;
   const float* src = partials + ((size_t)t * n_q_heads + h) * max_blocks * stride;
   float acc[kChanPerLane];
@@ -495,7 +539,8 @@ TL_EXPORT int tl_attention_generic(const void* q, int q_stride, void* out, int o
                                    const int32_t* positions, const int32_t* block_table, int bt_stride,
                                    int n_tokens, int n_q_heads, int n_kv_heads, int head_dim,
                                    int page_size, int window, float scale, float softcap, int chunk,
-                                   const float* sinks, int v_dim, int v_pitch, int dtype, hipStream_t stream) {
+                                   const float* sinks, int v_dim, int v_pitch, int dtype, int keep_first, int n_v_heads,
+                                   hipStream_t stream) {
   TL_REQUIRE(n_tokens >= 0 && n_q_heads > 0 && n_kv_heads > 0 && page_size > 0 && bt_stride > 0,
              "attention: bad sizes");
   TL_REQUIRE(n_q_heads % n_kv_heads == 0, "attention: %d query heads are not a multiple of %d kv heads",
@@ -505,6 +550,9 @@ TL_EXPORT int tl_attention_generic(const void* q, int q_stride, void* out, int o
   if (v_pitch <= 0) v_pitch = v_dim;  // value rows lie side by side
   TL_REQUIRE(v_pitch >= v_dim, "attention: value rows %d elements apart hold no %d channels", v_pitch, v_dim);
   TL_REQUIRE(window >= 0 && chunk >= 0, "attention: window=%d and chunk=%d must be >= 0", window, chunk);
+  TL_REQUIRE(keep_first >= 0, "attention: keep_first=%d must be >= 0", keep_first);
+  if (n_v_heads <= 0) n_v_heads = n_kv_heads;  // as many value heads as key heads
+  TL_REQUIRE(n_kv_heads % n_v_heads == 0, "attention: %d key heads are not a multiple of %d value heads", n_kv_heads, n_v_heads);
   if (v_dim <= 0 || v_dim > kMaxHeadDim)
     return tl_fail(TL_ERR_UNSUPPORTED, "attention: values of head size %d outside 1..%d", v_dim, kMaxHeadDim);
   if (n_tokens == 0) return TL_OK;
@@ -529,7 +577,7 @@ TL_EXPORT int tl_attention_generic(const void* q, int q_stride, void* out, int o
     attention_tile_kernel<T, VEC, CH><<<tgrid, kTileWaves * kWave, lds, stream>>>(                               \
         (const T*)q, q_stride, (T*)out, out_stride, (const T*)k_pages, (const T*)v_pages, token_seq, positions,  \
         block_table, bt_stride, n_tokens, n_q_heads, n_kv_heads, head_dim, page_size, window, scale, hb, softcap, \
-        chunk, sinks, v_dim, v_pitch);                                                                           \
+        chunk, sinks, v_dim, v_pitch, keep_first, n_v_heads);                                                    \
   } while (0)
 #define TL_TILE_LAUNCH(T, VEC)                                                                                   \
   do {                                                                                                           \
@@ -554,7 +602,8 @@ TL_EXPORT int tl_attention_generic(const void* q, int q_stride, void* out, int o
 #define TL_ATTN_LAUNCH(T, VEC)                                                                              \
   attention_generic_kernel<T, VEC><<<grid, kWavesPerBlock * kWave, 0, stream>>>(                            \
       (const T*)q, q_stride, (T*)out, out_stride, (const T*)k_pages, (const T*)v_pages, token_seq, positions, \
-      block_table, bt_stride, n_q_heads, n_kv_heads, head_dim, page_size, window, scale, softcap, chunk, sinks, v_dim, v_pitch)
+      block_table, bt_stride, n_q_heads, n_kv_heads, head_dim, page_size, window, scale, softcap, chunk, sinks, v_dim, v_pitch, \
+      keep_first, n_v_heads)
   if (dtype == TL_F32) {
     if (vec) TL_ATTN_LAUNCH(float, true);
     else TL_ATTN_LAUNCH(float, false);
@@ -578,7 +627,7 @@ TL_EXPORT int tl_attention_generic_split(const void* q, int q_stride, void* out,
                                          int n_tokens, int n_q_heads, int n_kv_heads, int head_dim,
                                          int page_size, int window, float scale, float softcap, int chunk,
                                          const float* sinks, int v_dim, int v_pitch, int dtype, int max_blocks,
-                                         float* partials, hipStream_t stream) {
+                                         float* partials, int keep_first, int n_v_heads, hipStream_t stream) {
   TL_REQUIRE(n_tokens >= 0 && n_q_heads > 0 && n_kv_heads > 0 && page_size > 0 && bt_stride > 0,
              "attention: bad sizes");
   TL_REQUIRE(n_q_heads % n_kv_heads == 0, "attention: %d query heads are not a multiple of %d kv heads",
@@ -588,6 +637,9 @@ TL_EXPORT int tl_attention_generic_split(const void* q, int q_stride, void* out,
   if (v_pitch <= 0) v_pitch = v_dim;  // value rows lie side by side
   TL_REQUIRE(v_pitch >= v_dim, "attention: value rows %d elements apart hold no %d channels", v_pitch, v_dim);
   TL_REQUIRE(window >= 0 && chunk >= 0, "attention: window=%d and chunk=%d must be >= 0", window, chunk);
+  TL_REQUIRE(keep_first >= 0, "attention: keep_first=%d must be >= 0", keep_first);
+  if (n_v_heads <= 0) n_v_heads = n_kv_heads;  // as many value heads as key heads
+  TL_REQUIRE(n_kv_heads % n_v_heads == 0, "attention: %d key heads are not a multiple of %d value heads", n_kv_heads, n_v_heads);
   if (v_dim <= 0 || v_dim > kMaxHeadDim)
     return tl_fail(TL_ERR_UNSUPPORTED, "attention: values of head size %d outside 1..%d", v_dim, kMaxHeadDim);
   TL_REQUIRE(max_blocks >= 1 && max_blocks <= 65535 && partials != nullptr, "attention: max_blocks=%d outside 1..65535, or no workspace", max_blocks);
@@ -601,11 +653,12 @@ TL_EXPORT int tl_attention_generic_split(const void* q, int q_stride, void* out,
   do {                                                                                                          \
     attention_blocks_kernel<T, VEC><<<grid, kWavesPerBlock * kWave, 0, stream>>>(                               \
         (const T*)q, q_stride, (const T*)k_pages, (const T*)v_pages, token_seq, positions, block_table, bt_stride, \
-        n_q_heads, n_kv_heads, head_dim, page_size, window, scale, partials, max_blocks, softcap, chunk, v_dim, v_pitch); \
+        n_q_heads, n_kv_heads, head_dim, page_size, window, scale, partials, max_blocks, softcap, chunk, v_dim, v_pitch,  \
+        keep_first, n_v_heads);                                                                                 \
     int rc = tl_check_launch("attention_blocks");                                                               \
     if (rc != TL_OK) return rc;                                                                                 \
     attention_join_kernel<T><<<grid_join, kWavesPerBlock * kWave, 0, stream>>>(                                 \
-        (T*)out, out_stride, positions, n_q_heads, v_dim, window, partials, max_blocks, chunk, sinks);         \
+        (T*)out, out_stride, positions, n_q_heads, v_dim, window, partials, max_blocks, chunk, sinks, keep_first); \
   } while (0)
   if (dtype == TL_F32) {
     if (vec) TL_ATTN_LAUNCH(float, true);

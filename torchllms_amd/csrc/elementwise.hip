@@ -386,22 +386,23 @@ TL_EXPORT int tl_rmsnorm_split(const void* x, const float* partial, int splits, 
 // The cosines and sines may come from a table [token][rotary_dim/2] of (cos, sin) made by
 // rope_table_kernel from the same positions (one table serves all layers of a step).
 __global__ void rope_table_kernel(const int32_t* __restrict__ positions, const float* __restrict__ inv_freq,
-                                  int n_tokens, int rot_half, float2* __restrict__ table) {
+                                  int n_tokens, int rot_half, float2* __restrict__ table, float magnitude) {
   const int idx = blockIdx.x * blockDim.x + threadIdx.x;
   if (idx >= n_tokens * rot_half) return;
   const int t = idx / rot_half;
   const int i = idx % rot_half;
   const float ang = (float)positions[t] * inv_freq[i];
-  table[idx] = make_float2(cosf(ang), sinf(ang));
+  // (a magnitude other than one is a factor on both, and so on the rotated channels: rescaled long contexts)
+  table[idx] = magnitude == 1.0f ? make_float2(cosf(ang), sinf(ang)) : make_float2(cosf(ang) * magnitude, sinf(ang) * magnitude);
 }
 
 TL_EXPORT int tl_rope_table(const int32_t* positions, const float* inv_freq, int n_tokens, int rot_half,
-                            float* table, hipStream_t stream) {
+                            float* table, float magnitude, hipStream_t stream) {
   TL_REQUIRE(n_tokens >= 0 && rot_half > 0, "rope_table: bad sizes");
   TL_REQUIRE((long long)n_tokens * rot_half < (1ll << 31), "rope_table: too many entries");
   if (n_tokens == 0) return TL_OK;
   const int total = n_tokens * rot_half;
-  rope_table_kernel<<<(total + 255) / 256, 256, 0, stream>>>(positions, inv_freq, n_tokens, rot_half, (float2*)table);
+  rope_table_kernel<<<(total + 255) / 256, 256, 0, stream>>>(positions, inv_freq, n_tokens, rot_half, (float2*)table, magnitude);
   return tl_check_launch("rope_table");
 }
 

@@ -11,10 +11,14 @@ __device__ __forceinline__ float sigmoid_r(float z) { return 1.0f / (1.0f + expf
 // ----------------------------------------------------------------------------- router
 // One wave a token.  z [n, z_stride]: 32-bit router outputs, the first n_out of a row.  s = softmax(z); the `top`
 // largest of s + correction are chosen (of equal ones the lower index), and the weights are their s.
+// correction may be null.  n_groups > 0: the outputs form that many equal groups of neighbours, a group's score is
+// the largest s in it, and only outputs of the keep_groups best groups (of equal ones the lower) can be chosen.
+// normalize: the weights are divided by their sum (+ 1e-20); then they are multiplied by route_scale.
 constexpr int kRouterPerLane = 8;  // outputs a lane holds: up to 512 experts
 __global__ void __launch_bounds__(256)
 router_topk_kernel(const float* __restrict__ z, int z_stride, const float* __restrict__ correction, int n, int n_out, int top,
-                   int32_t* __restrict__ ids, float* __restrict__ weights) {
+                   int32_t* __restrict__ ids, float* __restrict__ weights, int n_groups, int keep_groups, int normalize,
+                   float route_scale) {
   const int t = blockIdx.x * (blockDim.x / kWave) + threadIdx.x / kWave;
   const int lane = threadIdx.x % kWave;
   if (t >= n) return;
@@ -40,7 +44,39 @@ router_topk_kernel(const float* __restrict__ z, int z_stride, const float* __res
   for (int u = 0; u < kRouterPerLane; ++u) {
     const int e = lane + u * kWave;
     s[u] = s[u] / sum;
-    c[u] = e < n_out ? s[u] + correction[e] : -INFINITY;
+    c[u] = e < n_out ? (correction ? s[u] + correction[e] : s[u]) : -INFINITY;
+  }
+  if (n_groups > 0) {
+    const int per = n_out / n_groups;
+    float mine = -INFINITY;  // lane g: the score of group g (n_groups <= 64)
+    for (int g = 0; g < n_groups; ++g) {
+      float best = -INFINITY;
+#pragma unroll
+      for (int u = 0; u < kRouterPerLane; ++u) {
+        const int e = lane + u * kWave;
+        if (e < n_out && e / per == g) best = fmaxf(best, s[u]);
+      }
+      best = wave_max(best);
+      if (lane == g) mine = best;
+    }
+    unsigned long long open = 0ull;  // the groups that stay, one bit each
+    for (int k = 0; k < keep_groups; ++k) {
+      float best = mine;
+      int best_g = lane < n_groups ? lane : 0x7fffffff;
+#pragma unroll
+      for (int off = kWave / 2; off > 0; off >>= 1) {
+        const float ob = __shfl_xor(best, off, kWave);
+        const int og = __shfl_xor(best_g, off, kWave);
+        if (ob > best || (ob == best && og < best_g)) { best = ob; best_g = og; }
+      }
+      open |= 1ull << best_g;
+      if (lane == best_g) mine = -INFINITY;
+    }
+#pragma unroll
+    for (int u = 0; u < kRouterPerLane; ++u) {
+      const int e = lane + u * kWave;
+      if (e < n_out && !((open >> (e / per)) & 1ull)) c[u] = -INFINITY;
+    }
   }
   for (int k = 0; k < top; ++k) {
     float best = -INFINITY, best_s = 0.f;
@@ -63,6 +99,12 @@ router_topk_kernel(const float* __restrict__ z, int z_stride, const float* __res
 #pragma unroll
     for (int u = 0; u < kRouterPerLane; ++u)
       if (lane + u * kWave == best_e) c[u] = -INFINITY;
+  }
+  if ((normalize || route_scale != 1.0f) && lane == 0) {  // (the lane that wrote them reads them back)
+    float* w = weights + (size_t)t * top;
+    float total = 0.f;
+    for (int k = 0; k < top; ++k) total += w[k];
+    for (int k = 0; k < top; ++k) w[k] = (normalize ? w[k] / (total + 1e-20f) : w[k]) * route_scale;
   }
 }
 
@@ -387,7 +429,7 @@ expert_combine_kernel(const YT* __restrict__ y, const int32_t* __restrict__ pos,
   const int t = blockIdx.x;
   const int d = blockIdx.y * blockDim.x + threadIdx.x;
   if (d >= D) return;
-  const float share = shared ? sigmoid_r(sg[(size_t)t * sg_stride]) : 0.f;
+  const float share = shared ? (sg ? sigmoid_r(sg[(size_t)t * sg_stride]) : 1.f) : 0.f;  // (no gate: added as it is)
   float total = 0.f;
   for (int j = 0; j < top; ++j) {
     const int e = ids[(size_t)t * top + j];
@@ -510,13 +552,17 @@ post_norm_add_norm_held_kernel(float* __restrict__ stream, const T* __restrict__
 
 // ============================================================================= C interface
 TL_EXPORT int tl_router_topk(const float* z, int z_stride, const float* correction, int n, int n_out, int top, int32_t* ids,
-                             float* weights, hipStream_t stream) {
+                             float* weights, int n_groups, int keep_groups, int normalize, float route_scale, hipStream_t stream) {
   TL_REQUIRE(n >= 0 && n_out > 0 && top > 0 && top <= n_out && z_stride >= n_out, "router_topk: bad sizes");
+  TL_REQUIRE(n_groups >= 0 && (n_groups == 0 || (n_groups <= kWave && n_out % n_groups == 0 && keep_groups > 0 && keep_groups <= n_groups
+                                                 && (long long)keep_groups * (n_out / n_groups) >= top)),
+             "router_topk: %d groups of which %d stay do not fit %d outputs and %d choices (at most 64 groups)", n_groups, keep_groups, n_out, top);
   if (n_out > kRouterPerLane * kWave)
     return tl_fail(TL_ERR_UNSUPPORTED, "router_topk: %d router outputs, at most %d", n_out, kRouterPerLane * kWave);
   if (n == 0) return TL_OK;
   const int per_block = 256 / kWave;
-  router_topk_kernel<<<(n + per_block - 1) / per_block, 256, 0, stream>>>(z, z_stride, correction, n, n_out, top, ids, weights);
+  router_topk_kernel<<<(n + per_block - 1) / per_block, 256, 0, stream>>>(z, z_stride, correction, n, n_out, top, ids, weights, n_groups,
+                                                                         keep_groups, normalize, route_scale);
   return tl_check_launch("router_topk");
 }
 
@@ -613,7 +659,6 @@ TL_EXPORT int tl_expert_combine(const void* y, int y_f32, const int32_t* pos, co
                                 int n_experts, const void* x, const void* shared, const float* sg, int sg_stride, void* out, int n,
                                 int D, int dtype, hipStream_t stream) {
   TL_REQUIRE(n >= 0 && n <= 0x7fffffff && top > 0 && n_experts >= 0 && D > 0 && (D + 255) / 256 <= 65535, "expert_combine: bad sizes");
-  TL_REQUIRE(shared == nullptr || sg != nullptr, "expert_combine: a shared expert without its gate");
   if (n == 0) return TL_OK;
   const dim3 cgrid(n, (D + 255) / 256);
 #define TL_COMBINE(T, YT)                                                                                                   \

@@ -488,6 +488,7 @@ scan_carry_kernel(float* __restrict__ ws, const float* __restrict__ seg_dt, cons
 // tile is worked on; in LDS the keys and queries are made unit vectors once per tile; then the tile's
 // tokens follow each other without a barrier (sums over a column's lanes by lane-to-lane moves).
 constexpr int kDeltaTile = 16;
+__device__ __forceinline__ float log_sigmoid_f(float z) { return fminf(z, 0.f) - log1pf(expf(-fabsf(z))); }
 // kDeltaCols, a template argument: 16 or 32 columns a block.  The time of a token is the block's multiply-adds, so
 // a launch of few blocks (a prompt of one request: heads * dv / 16 blocks, 256 for 32 heads of 128 columns) takes 16;
 // a launch that fills the GPU anyway (decode steps of many requests) takes 32 and has half the blocks to start.
@@ -519,7 +520,10 @@ __device__ __forceinline__ float row_group_sum(float v, int width) {
 // CH: a decay of its own for every key channel (row of S) of a head: the pre-activations come as 32-bit rows
 // a_ch [n_tokens, a_stride] with H * dk columns, dt_bias has H * dk entries, and a token's decays lie in LDS beside
 // its key; the column a_off of proj is not read.
-template <typename T, bool VEC, int kDeltaRows, int kDeltaCols, bool CH>
+// RULE 0: the delta rule with a decay per head; 1: with a decay per key channel (CH); 2: no delta and no unit
+// vectors, S <- diag(decay) S + k v^T with q times dk^-1/2 and decay = sigmoid(a_ch + dt_bias)^plain_rate per key
+// channel (gated linear attention; proj and A_log are not read).
+template <typename T, bool VEC, int kDeltaRows, int kDeltaCols, int RULE>
 // (Held to 128 registers, so that more of a decode step's many short blocks share a CU, the compiler spills 400 to
 // 1,000 bytes a lane: what the tile's pipeline carries is more than that.  It is left its 233 to 256.)
 __global__ void __launch_bounds__(512)
@@ -527,7 +531,8 @@ gated_delta_kernel(const T* __restrict__ qkv, int qkv_stride, const T* __restric
                    int a_off, const float* __restrict__ A_log, const float* __restrict__ dt_bias,
                    float* __restrict__ state, long long state_stride, const int32_t* __restrict__ qo_indptr,
                    const int32_t* __restrict__ slot_ids, float* __restrict__ o_raw, int H, int G, int dk, int dv, int lpc,
-                   int col_groups, const float* __restrict__ a_ch, int a_stride) {
+                   int col_groups, const float* __restrict__ a_ch, int a_stride, float plain_rate) {
+  constexpr bool CH = RULE >= 1, PLAIN = RULE == 2;
   extern __shared__ __attribute__((aligned(16))) float lds[];
   // per token of the tile: k [dk], q [dk] (raw, then unit), v [kDeltaCols], o [kDeltaCols]; then six scalars
   const int dkp = dk + dk / 16 * 4;  // a token's keys in LDS: four floats of padding after every sixteen, so that
@@ -560,7 +565,7 @@ gated_delta_kernel(const T* __restrict__ qkv, int qkv_stride, const T* __restric
 #pragma unroll
     for (int r = 0; r < kDeltaRows; ++r) S[r] = i0 + r < dk ? st[i0 + r] : 0.f;
   }
-  const float neg_rate = -expf(A_log[h]), bias = CH ? 0.f : dt_bias[h];
+  const float neg_rate = PLAIN ? 0.f : -expf(A_log[h]), bias = CH ? 0.f : dt_bias[h];
   const float q_scale = 1.0f / sqrtf((float)dk);
   const int q_col = g * dk, k_col = G * dk + g * dk, v_col = 2 * G * dk + h * dv + cg * kDeltaCols;
   const int v_cols = min(kDeltaCols, dv - cg * kDeltaCols);
@@ -576,7 +581,7 @@ gated_delta_kernel(const T* __restrict__ qkv, int qkv_stride, const T* __restric
   T pre_kq[kPreKQ], pre_v[kPreV], pre_b = from_f32<T>(0.f), pre_a = from_f32<T>(0.f);
   auto fetch = [&](int t0) {
     const int nt = min(kDeltaTile, end - t0);
-    if (threadIdx.x < nt) {
+    if (!PLAIN && threadIdx.x < nt) {
       const T* pr = proj + (size_t)(t0 + threadIdx.x) * proj_stride;
       pre_b = pr[b_off + h];
       if (!CH) pre_a = pr[a_off + h];
@@ -618,14 +623,14 @@ gated_delta_kernel(const T* __restrict__ qkv, int qkv_stride, const T* __restric
       if (tt < nt && d < v_cols) v_l[tt * kDeltaCols + d] = to_f32(pre_v[u]);
     }
     if (threadIdx.x < nt) {
-      sc_l[6 * threadIdx.x] = sigmoid_f(to_f32(pre_b));
+      sc_l[6 * threadIdx.x] = PLAIN ? 1.f : sigmoid_f(to_f32(pre_b));
       if (!CH) sc_l[6 * threadIdx.x + 1] = expf(neg_rate * softplus_f(to_f32(pre_a) + bias));
     }
     if (CH) {
       for (int e = threadIdx.x; e < nt * dk; e += n_threads) {
         const int tt = e / dk, d = e % dk;
         const float pre = a_ch[(size_t)(t0 + tt) * a_stride + h * dk + d] + dt_bias[h * dk + d];
-        g_l[tt * dkp + d + d / 16 * 4] = expf(neg_rate * softplus_f(pre));
+        g_l[tt * dkp + d + d / 16 * 4] = PLAIN ? expf(plain_rate * log_sigmoid_f(pre)) : expf(neg_rate * softplus_f(pre));
       }
     }
     if (t0 + kDeltaTile < end) fetch(t0 + kDeltaTile);  // on its way while this tile is worked on
@@ -647,7 +652,7 @@ gated_delta_kernel(const T* __restrict__ qkv, int qkv_stride, const T* __restric
       qq2 = row_group_sum(qq2, 8);
       kq = row_group_sum(kq, 8);
       if (tt < nt && sub == 0) {
-        const float k_inv = 1.0f / sqrtf(kk2 + 1e-6f), q_inv = q_scale / sqrtf(qq2 + 1e-6f);
+        const float k_inv = PLAIN ? 1.f : 1.0f / sqrtf(kk2 + 1e-6f), q_inv = PLAIN ? q_scale : q_scale / sqrtf(qq2 + 1e-6f);
         sc_l[6 * tt + 2] = k_inv;
         sc_l[6 * tt + 3] = q_inv;
         sc_l[6 * tt + 4] = kq * k_inv * q_inv;  // k^ . q^
@@ -716,7 +721,7 @@ gated_delta_kernel(const T* __restrict__ qkv, int qkv_stride, const T* __restric
       if (lpc >= 4) { kv_all += dpp_xor2(kv_all); sq_all += dpp_xor2(sq_all); }
       if (lpc >= 8) { kv_all += dpp_half_mirror(kv_all); sq_all += dpp_half_mirror(sq_all); }
       if (lpc >= 16) { kv_all += dpp_mirror(kv_all); sq_all += dpp_mirror(sq_all); }
-      const float u = x.beta * (x.v - kv_all);
+      const float u = PLAIN ? x.v : x.beta * (x.v - kv_all);
       if (live && part == 0) o_l[tt * kDeltaCols + j_loc] = fmaf(u, x.kq, sq_all);
 #pragma unroll
       for (int r = 0; r < kDeltaRows; ++r) S[r] = fmaf(x.kk[r], u, S[r]);
@@ -755,13 +760,14 @@ gated_delta_kernel(const T* __restrict__ qkv, int qkv_stride, const T* __restric
 // ahead, few registers, so that many of these short blocks share a CU.  Every sum is taken in the order in which
 // gated_delta_kernel takes it (the norms by eight lanes over every eighth channel, the products with the state by
 // four chains a lane and then the column's lanes), so a token's result has the same bits from either kernel.
-template <typename T, bool VEC, int kDeltaRows, bool CH>
+template <typename T, bool VEC, int kDeltaRows, int RULE>
 __global__ void __launch_bounds__(512)
 gated_delta_step_kernel(const T* __restrict__ qkv, int qkv_stride, const T* __restrict__ proj, int proj_stride, int b_off,
                         int a_off, const float* __restrict__ A_log, const float* __restrict__ dt_bias,
                         float* __restrict__ state, long long state_stride, const int32_t* __restrict__ qo_indptr,
                         const int32_t* __restrict__ slot_ids, float* __restrict__ o_raw, int H, int G, int dk, int dv,
-                        int lpc, int col_groups, const float* __restrict__ a_ch, int a_stride) {
+                        int lpc, int col_groups, const float* __restrict__ a_ch, int a_stride, float plain_rate) {
+  constexpr bool CH = RULE >= 1, PLAIN = RULE == 2;
   constexpr int kCols = 32;
   extern __shared__ __attribute__((aligned(16))) float lds[];
   const int dkp = dk + dk / 16 * 4;
@@ -783,9 +789,11 @@ gated_delta_step_kernel(const T* __restrict__ qkv, int qkv_stride, const T* __re
   }
   float* g_l = lds + 2 * dkp;  // (CH) the token's decays, once for all columns of the block
   if (CH) {
-    const float rate = -expf(A_log[h]);
-    for (int d = threadIdx.x; d < dk; d += blockDim.x)
-      g_l[d + d / 16 * 4] = expf(rate * softplus_f(a_ch[t * a_stride + h * dk + d] + dt_bias[h * dk + d]));
+    const float rate = PLAIN ? 0.f : -expf(A_log[h]);
+    for (int d = threadIdx.x; d < dk; d += blockDim.x) {
+      const float pre = a_ch[t * a_stride + h * dk + d] + dt_bias[h * dk + d];
+      g_l[d + d / 16 * 4] = PLAIN ? expf(plain_rate * log_sigmoid_f(pre)) : expf(rate * softplus_f(pre));
+    }
   }
   float* st = state + (long long)slot_ids[row] * state_stride + ((size_t)h * dv + j) * dk;
   float S[kDeltaRows];
@@ -800,8 +808,8 @@ gated_delta_step_kernel(const T* __restrict__ qkv, int qkv_stride, const T* __re
     for (int r = 0; r < kDeltaRows; ++r) S[r] = i0 + r < dk ? st[i0 + r] : 0.f;
   }
   const float v = to_f32(tok[2 * G * dk + h * dv + j]);
-  const float pb = to_f32(proj[t * proj_stride + b_off + h]), pa = CH ? 0.f : to_f32(proj[t * proj_stride + a_off + h]);
-  const float neg_rate = -expf(A_log[h]), bias = CH ? 0.f : dt_bias[h];
+  const float pb = PLAIN ? 0.f : to_f32(proj[t * proj_stride + b_off + h]), pa = CH ? 0.f : to_f32(proj[t * proj_stride + a_off + h]);
+  const float neg_rate = PLAIN ? 0.f : -expf(A_log[h]), bias = CH ? 0.f : dt_bias[h];
   __syncthreads();
   const int sub = threadIdx.x % 8;
   float kk2 = 0.f, qq2 = 0.f, kq = 0.f;
@@ -814,7 +822,8 @@ gated_delta_step_kernel(const T* __restrict__ qkv, int qkv_stride, const T* __re
   kk2 = row_group_sum(kk2, 8);
   qq2 = row_group_sum(qq2, 8);
   kq = row_group_sum(kq, 8);
-  const float k_inv = 1.0f / sqrtf(kk2 + 1e-6f), q_inv = (1.0f / sqrtf((float)dk)) / sqrtf(qq2 + 1e-6f);
+  const float k_inv = PLAIN ? 1.f : 1.0f / sqrtf(kk2 + 1e-6f);
+  const float q_inv = PLAIN ? 1.0f / sqrtf((float)dk) : (1.0f / sqrtf((float)dk)) / sqrtf(qq2 + 1e-6f);
   const float kq_hat = kq * k_inv * q_inv;
   const float beta = sigmoid_f(pb), decay = CH ? 0.f : expf(neg_rate * softplus_f(pa + bias));
   float kv[4] = {0.f, 0.f, 0.f, 0.f}, sq[4] = {0.f, 0.f, 0.f, 0.f};
@@ -833,7 +842,7 @@ gated_delta_step_kernel(const T* __restrict__ qkv, int qkv_stride, const T* __re
   }
   const float kv_all = row_group_sum((kv[0] + kv[1]) + (kv[2] + kv[3]), lpc);
   const float sq_all = row_group_sum((sq[0] + sq[1]) + (sq[2] + sq[3]), lpc);
-  const float u = beta * (v - kv_all);
+  const float u = PLAIN ? v : beta * (v - kv_all);
   if (live && part == 0) o_raw[(t * H + h) * dv + j] = fmaf(u, kq_hat, sq_all);
 #pragma unroll
   for (int r = 0; r < kDeltaRows; ++r) S[r] = fmaf(kk[r], u, S[r]);
@@ -1095,7 +1104,7 @@ TL_EXPORT int tl_gated_delta(const void* qkv, int qkv_stride, const void* proj, 
                              int a_off, const float* A_log, const float* dt_bias, const float* norm_w, float eps, float* state,
                              long long state_stride, const int32_t* qo_indptr, const int32_t* slot_ids, void* out, int n_tokens,
                              int n_seqs, int H, int G, int dk, int dv, float* o_raw, int dtype, const void* gate, int gate_stride,
-                             int gate_sigmoid, const float* a_ch, int a_stride, hipStream_t stream) {
+                             int gate_sigmoid, const float* a_ch, int a_stride, float plain_rate, hipStream_t stream) {
   TL_REQUIRE(n_seqs >= 0 && n_tokens >= 0 && H > 0 && G > 0 && dk > 0 && dv > 0, "gated_delta: bad sizes");
   TL_REQUIRE(H % G == 0, "gated_delta: %d heads are not a multiple of %d key heads", H, G);
   if (dk > 256) return tl_fail(TL_ERR_UNSUPPORTED, "gated_delta: keys of %d channels, at most 256", dk);
@@ -1110,6 +1119,9 @@ TL_EXPORT int tl_gated_delta(const void* qkv, int qkv_stride, const void* proj, 
   // columns a block: 16 while that leaves fewer than two blocks a CU, else 32 (a step of single tokens: always 32)
   const bool single = n_tokens == n_seqs;
   const bool ch = a_ch != nullptr;
+  const bool plain = plain_rate > 0.f;
+  TL_REQUIRE(!plain || ch, "gated_delta: the plain rule has a decay per key channel");
+  TL_REQUIRE(plain || (A_log != nullptr && proj != nullptr), "gated_delta: no A_log or no projections");
   const int cols = !single && (long long)n_seqs * H * ((dv + 15) / 16) < 2LL * tl_device_facts().compute_units ? 16 : 32;
   const int threads = (cols * lpc + kWave - 1) / kWave * kWave;
   const int col_groups = (dv + cols - 1) / cols;
@@ -1119,7 +1131,7 @@ TL_EXPORT int tl_gated_delta(const void* qkv, int qkv_stride, const void* proj, 
 #define TL_DELTA_R(T, VEC, R, C, CH)                                                                                   \
   gated_delta_kernel<T, VEC, R, C, CH><<<grid, threads, lds, stream>>>(                                                \
       (const T*)qkv, qkv_stride, (const T*)proj, proj_stride, b_off, a_off, A_log, dt_bias, state, state_stride,       \
-      qo_indptr, slot_ids, o_raw, H, G, dk, dv, lpc, col_groups, a_ch, a_stride)
+      qo_indptr, slot_ids, o_raw, H, G, dk, dv, lpc, col_groups, a_ch, a_stride, plain_rate)
 #define TL_DELTA(T, VEC, CH)                                      \
   do {                                                            \
     if (rows == 8 && cols == 16) TL_DELTA_R(T, VEC, 8, 16, CH);   \
@@ -1135,11 +1147,11 @@ TL_EXPORT int tl_gated_delta(const void* qkv, int qkv_stride, const void* proj, 
     if (rows == 8)                                                                                                     \
       gated_delta_step_kernel<T, VEC, 8, CH><<<grid, threads, step_lds, stream>>>(                                     \
           (const T*)qkv, qkv_stride, (const T*)proj, proj_stride, b_off, a_off, A_log, dt_bias, state, state_stride,   \
-          qo_indptr, slot_ids, o_raw, H, G, dk, dv, lpc, col_groups, a_ch, a_stride);                                  \
+          qo_indptr, slot_ids, o_raw, H, G, dk, dv, lpc, col_groups, a_ch, a_stride, plain_rate);                      \
     else                                                                                                               \
       gated_delta_step_kernel<T, VEC, 16, CH><<<grid, threads, step_lds, stream>>>(                                    \
           (const T*)qkv, qkv_stride, (const T*)proj, proj_stride, b_off, a_off, A_log, dt_bias, state, state_stride,   \
-          qo_indptr, slot_ids, o_raw, H, G, dk, dv, lpc, col_groups, a_ch, a_stride);                                  \
+          qo_indptr, slot_ids, o_raw, H, G, dk, dv, lpc, col_groups, a_ch, a_stride, plain_rate);                      \
   } while (0)
 #define TL_DELTA_ANY(T, VEC, CH)          \
   do {                                    \
@@ -1148,10 +1160,12 @@ TL_EXPORT int tl_gated_delta(const void* qkv, int qkv_stride, const void* proj, 
   } while (0)
 #define TL_DELTA_T(T)                            \
   do {                                           \
-    if (vec && ch) TL_DELTA_ANY(T, true, true);  \
-    else if (vec) TL_DELTA_ANY(T, true, false);  \
-    else if (ch) TL_DELTA_ANY(T, false, true);   \
-    else TL_DELTA_ANY(T, false, false);          \
+    if (vec && plain) TL_DELTA_ANY(T, true, 2);  \
+    else if (plain) TL_DELTA_ANY(T, false, 2);   \
+    else if (vec && ch) TL_DELTA_ANY(T, true, 1);  \
+    else if (vec) TL_DELTA_ANY(T, true, 0);      \
+    else if (ch) TL_DELTA_ANY(T, false, 1);      \
+    else TL_DELTA_ANY(T, false, 0);              \
   } while (0)
   if (dtype == TL_F32) TL_DELTA_T(float);
   else TL_DELTA_T(bf16_t);
@@ -1186,7 +1200,6 @@ TL_EXPORT int tl_gated_delta(const void* qkv, int qkv_stride, const void* proj, 
 namespace {
 constexpr int kMemCols = 32;
 
-__device__ __forceinline__ float log_sigmoid_f(float z) { return fminf(z, 0.f) - log1pf(expf(-fabsf(z))); }
 
 template <typename T, bool VEC, int R>
 __global__ void __launch_bounds__(512)

@@ -304,7 +304,8 @@ class Engine:
                 # the last step's advance gave back the pages that the window has passed: their
                 # blocks are -1 in the requests' tables, and so they are here
                 first_live = np.maximum(positions - window + 1, 0) // page
-                released = np.arange(bt.shape[1], dtype=np.int64)[None, :] < first_live[:, None]
+                blocks = np.arange(bt.shape[1], dtype=np.int64)[None, :]
+                released = (blocks < first_live[:, None]) & (blocks >= cache.kept_blocks(g))  # (blocks of kept first positions stay)
                 if (released & (bt >= 0)).any():
                     bt = np.where(released, np.int32(-1), bt)
             tables.append(bt)

@@ -161,12 +161,13 @@ class Scheduler:
         """The pages of ``group`` that a request of ``n_tokens`` cannot do without.  A group that
         keeps every key needs them all; a group with a window gives pages back as the window passes
         them, and a portion can be cut down to one token, so what it must hold at once are the
-        pages that ``window`` keys touch (one more when they straddle a page's edge)."""
+        pages that ``window`` keys touch (one more when they straddle a page's edge), and those of the first positions
+        that stay visible behind the window, if the group keeps any."""
         whole = self.cache.blocks_for(n_tokens, group)
         window = self.cache.groups[group].window
         if window <= 0:
             return whole
-        return min(whole, self.cache.blocks_for(window, group) + 1)
+        return min(whole, self.cache.blocks_for(window, group) + 1 + self.cache.kept_blocks(group))
 
     # ------------------------------------------------------------------ planning
     def _pages_for(self, req: Request, n_new: int) -> List[int]:

@@ -32,17 +32,24 @@ def paged_attention(
     v_head_dim=None,
     values_in_keys: bool = False,
     value_offset: int = 0,
+    keep_first: int = 0,
+    value_heads=None,
 ) -> torch.Tensor:
     """Attention of this step's queries (first Hq * dh columns of ``qkv``) over their requests'
     cached keys and values; returns [n_tokens, Hq * dv].  Capped scores (``softcap``), chunks
     (``chunk``) and sinks are every kernel's; values of another head size than the keys, or values that are
-    channels of the key rows (``values_in_keys``, from ``value_offset`` on), are the plain kernel's alone."""
+    channels of the key rows (``values_in_keys``, from ``value_offset`` on), first keys that stay visible behind a
+    window (``keep_first``) and values with fewer heads than the keys (``value_heads``) are the plain kernel's alone."""
     n = qkv.shape[0]
     n_dec = ctx.host.n_decode
     v_dim = head_dim if v_head_dim is None else int(v_head_dim)
-    plain_only = v_dim != head_dim or values_in_keys  # (the MFMA kernels take a cap, chunks and sinks, but one head size)
+    kept = keep_first if window > 0 or chunk > 0 else 0  # (without a window every key is seen anyway)
+    fewer_values = value_heads is not None and value_heads != n_kv_heads
+    # (the MFMA kernels take a cap, chunks and sinks, but one head size, one range of keys and as many value heads as key heads)
+    plain_only = v_dim != head_dim or values_in_keys or kept > 0 or fewer_values
     extended = softcap > 0 or chunk > 0 or sinks is not None or plain_only
-    extras = dict(softcap=softcap, chunk=chunk, sinks=sinks, v_head_dim=v_dim, values_in_keys=values_in_keys, value_offset=value_offset) if extended else {}
+    extras = dict(softcap=softcap, chunk=chunk, sinks=sinks, v_head_dim=v_dim, values_in_keys=values_in_keys, value_offset=value_offset,
+                  keep_first=kept, value_heads=value_heads) if extended else {}
     fast_extras = dict(softcap=softcap, chunk=chunk, sinks=sinks) if extended else {}
     fast_decode = not plain_only and n_dec > 0 and ops.decode_attention_supported(qkv.dtype, n_q_heads, n_kv_heads, head_dim)
     # the MFMA prefill kernel takes positive softmax scales only; anything else runs the plain kernel
@@ -74,6 +81,7 @@ def paged_attention(
                 longest = min(longest, window)
             if chunk > 0:
                 longest = min(longest, chunk)
+            # (kept first keys come as blocks of their own, which the split form counts by itself)
             plain = ops.attention_generic_split if longest > GENERIC_SPLIT_FROM else ops.attention_generic
             extra = dict(longest=longest) if longest > GENERIC_SPLIT_FROM else {}
             plain(

@@ -33,11 +33,14 @@ ATTENTION_MAX_KEY_DIM = 1024
 
 
 def _generic_arguments(qkv, n_q_heads, n_kv_heads, head_dim, k_pages, v_pages, token_seq, positions, block_table, out,
-                       sinks=None, v_head_dim=None, values_in_keys=False, value_offset=0):
+                       sinks=None, v_head_dim=None, values_in_keys=False, value_offset=0, keep_first=0, value_heads=None):
     """What both launches of the plain kernel ask of their arguments; returns (tokens, page size, out, value head
     size, elements between two value rows).  ``values_in_keys``: a token's value is the first ``v_head_dim`` channels
     of its key row, and ``v_pages`` is ``k_pages``; ``value_offset``: it is the ``v_head_dim`` channels from there on."""
     v_dim = head_dim if v_head_dim is None else int(v_head_dim)
+    n_v_heads = n_kv_heads if value_heads is None else int(value_heads)
+    if keep_first < 0 or n_v_heads <= 0 or n_kv_heads % n_v_heads or (values_in_keys and n_v_heads != n_kv_heads):
+        raise KernelError(f"attention: keep_first={keep_first} must not be negative, and {n_kv_heads} key heads must be a multiple of {n_v_heads} value heads")
     if values_in_keys and (v_pages.data_ptr() != k_pages.data_ptr() or v_pages.shape != k_pages.shape or value_offset < 0 or value_offset + v_dim > head_dim):
         raise KernelError("attention: values inside the keys are the keys' own pages and lie inside the key rows")
     if value_offset and not values_in_keys:
@@ -55,8 +58,8 @@ def _generic_arguments(qkv, n_q_heads, n_kv_heads, head_dim, k_pages, v_pages, t
     if block_table.dim() != 2 or block_table.dtype != torch.int32 or block_table.stride(1) != 1:
         raise KernelError("attention: block_table must be an int32 matrix")
     page_size = k_pages.shape[2]
-    for pg, width in ((k_pages, head_dim), (v_pages, head_dim if values_in_keys else v_dim)):
-        if pg.dim() != 4 or pg.shape[1:] != (n_kv_heads, page_size, width) or pg.dtype != qkv.dtype or not pg.is_contiguous():
+    for pg, heads, width in ((k_pages, n_kv_heads, head_dim), (v_pages, n_v_heads, head_dim if values_in_keys else v_dim)):
+        if pg.dim() != 4 or pg.shape[1:] != (heads, page_size, width) or pg.dtype != qkv.dtype or not pg.is_contiguous():
             raise KernelError("attention: pages must be contiguous [pages, Hkv, page_size, head size] of the query's dtype")
     if k_pages.shape[0] != v_pages.shape[0]:
         raise KernelError("attention: key and value pools differ in their number of pages")
@@ -86,22 +89,28 @@ def attention_generic(
     v_head_dim: Optional[int] = None,
     values_in_keys: bool = False,
     value_offset: int = 0,
+    keep_first: int = 0,
+    value_heads: Optional[int] = None,
 ) -> torch.Tensor:
     """Attention of each token's query heads (the first Hq * dh columns of ``qkv``) over the paged
     keys and values of its request; returns [n, Hq * dv].  ``softcap`` c > 0: scores become
     c * tanh(score / c).  ``chunk`` > 0: a query sees only the keys of its own chunk of that many
     positions.  ``sinks``: one 32-bit number per query head whose exponential joins the softmax's
     denominator.  ``v_head_dim``: the values' head size when it is not the keys'.  ``values_in_keys``: a
-    token's value is ``v_head_dim`` channels of its key row, from ``value_offset`` on (``v_pages`` is ``k_pages``)."""
+    token's value is ``v_head_dim`` channels of its key row, from ``value_offset`` on (``v_pages`` is ``k_pages``).
+    ``keep_first`` n > 0: behind a window a query also sees the first n positions of its request.  ``value_heads``:
+    the value pages have fewer heads than the key pages, and key head g reads value head ``g % value_heads``
+    (several score maps over the same values: the key heads of map m are ``m * value_heads ..``)."""
     n, page_size, out, v_dim, v_pitch = _generic_arguments(qkv, n_q_heads, n_kv_heads, head_dim, k_pages, v_pages, token_seq,
-                                                           positions, block_table, out, sinks, v_head_dim, values_in_keys, value_offset)
+                                                           positions, block_table, out, sinks, v_head_dim, values_in_keys, value_offset,
+                                                           keep_first, value_heads)
     v_at = v_pages.data_ptr() + int(value_offset) * v_pages.element_size()
     check(
         core().tl_attention_generic(
             qkv.data_ptr(), qkv.stride(0), out.data_ptr(), out.stride(0), k_pages.data_ptr(), v_at,
             token_seq.data_ptr(), positions.data_ptr(), block_table.data_ptr(), block_table.stride(0), n,
             n_q_heads, n_kv_heads, head_dim, page_size, window, float(scale), float(softcap), int(chunk), _ptr(sinks), v_dim,
-            v_pitch, dtype_code(qkv.dtype), _stream(),
+            v_pitch, dtype_code(qkv.dtype), int(keep_first), int(value_heads or 0), _stream(),
         )
     )
     return out
@@ -129,23 +138,26 @@ def attention_generic_split(
     v_head_dim: Optional[int] = None,
     values_in_keys: bool = False,
     value_offset: int = 0,
+    keep_first: int = 0,
+    value_heads: Optional[int] = None,
 ) -> torch.Tensor:
     """``attention_generic`` for steps with few tokens and long contexts (decode): every block of 64
     keys is computed by a wave of its own and a second kernel joins the blocks in order.  The same
     blocks, operations and order as the one-wave form: the same bits.  ``longest``: an upper bound of
     the keys any token sees (its position + 1, or the window)."""
     n, page_size, out, v_dim, v_pitch = _generic_arguments(qkv, n_q_heads, n_kv_heads, head_dim, k_pages, v_pages, token_seq,
-                                                           positions, block_table, out, sinks, v_head_dim, values_in_keys, value_offset)
+                                                           positions, block_table, out, sinks, v_head_dim, values_in_keys, value_offset,
+                                                           keep_first, value_heads)
     v_at = v_pages.data_ptr() + int(value_offset) * v_pages.element_size()
     # blocks are aligned to absolute positions: a range of `longest` keys touches at most this many
-    max_blocks = max(int(longest), 1) // 64 + 2
+    max_blocks = max(int(longest), 1) // 64 + 2 + (int(keep_first) + 63) // 64
     partials = torch.empty((n, n_q_heads, max_blocks, v_dim + 2), dtype=torch.float32, device=qkv.device)
     check(
         core().tl_attention_generic_split(
             qkv.data_ptr(), qkv.stride(0), out.data_ptr(), out.stride(0), k_pages.data_ptr(), v_at,
             token_seq.data_ptr(), positions.data_ptr(), block_table.data_ptr(), block_table.stride(0), n,
             n_q_heads, n_kv_heads, head_dim, page_size, window, float(scale), float(softcap), int(chunk), _ptr(sinks), v_dim,
-            v_pitch, dtype_code(qkv.dtype), max_blocks, partials.data_ptr(), _stream(),
+            v_pitch, dtype_code(qkv.dtype), max_blocks, partials.data_ptr(), int(keep_first), int(value_heads or 0), _stream(),
         )
     )
     return out

@@ -38,6 +38,7 @@ CORE_SOURCES = [
     "sequence_ops.hip",
     "head_ops.hip",
     "routed_ops.hip",
+    "stream_ops.hip",
 ]
 HEADERS = ["common.h", "qkv_epilogue.h", "no_alloc.h"]
 

@@ -111,16 +111,16 @@ def _rmsnorm_split(x, weight, eps, delta: "SplitSums", rows, return_sum):
     return (h_out, y) if return_sum else y
 
 
-def rope_table(positions: torch.Tensor, inv_freq: torch.Tensor) -> torch.Tensor:
+def rope_table(positions: torch.Tensor, inv_freq: torch.Tensor, magnitude: float = 1.0) -> torch.Tensor:
     """float32 [n, len(inv_freq), 2]: cosine and sine of ``float(position) * inv_freq`` (32-bit angle,
-    precise functions).  One table serves every layer of a step that rotates alike."""
+    precise functions), both times ``magnitude``.  One table serves every layer of a step that rotates alike."""
     _gpu(positions, inv_freq)
     _i32(positions, "positions")
     if inv_freq.dtype != torch.float32 or inv_freq.dim() != 1 or not inv_freq.is_contiguous() or inv_freq.numel() == 0:
         raise KernelError("inv_freq must be a contiguous float32 vector")
     n, half = positions.numel(), inv_freq.numel()
     out = torch.empty((n, half, 2), dtype=torch.float32, device=positions.device)
-    check(core().tl_rope_table(positions.data_ptr(), inv_freq.data_ptr(), n, half, out.data_ptr(), _stream()))
+    check(core().tl_rope_table(positions.data_ptr(), inv_freq.data_ptr(), n, half, out.data_ptr(), float(magnitude), _stream()))
     return out
 
 

@@ -28,21 +28,24 @@ _CORE_SIGNATURES = {
     "tl_embed": [_P, _P, _P, _I, _I, _I, _P],
     "tl_rmsnorm": [_P, _P, _P, _P, _I, _P, _P, _I, _I, _F, _I, _P],
     "tl_rmsnorm_split": [_P, _P, _I, _I64, _P, _P, _I, _P, _P, _I, _I, _F, _P],
-    "tl_rope_table": [_P, _P, _I, _I, _P, _P],
+    "tl_rope_table": [_P, _P, _I, _I, _P, _F, _P],
     "tl_rope_kv_write": [_P, _I, _I, _I, _I, _P, _P, _P, _I, _I, _P, _P, _P, _I, _I, _P],
     "tl_silu_mul": [_P, _P, _I, _I, _I, _P],
     "tl_add_bias": [_P, _P, _I, _I, _I, _I, _P],
-    "tl_attention_generic": [_P, _I, _P, _I, _P, _P, _P, _P, _P, _I, _I, _I, _I, _I, _I, _I, _F, _F, _I, _P, _I, _I, _I, _P],
-    "tl_attention_generic_split": [_P, _I, _P, _I, _P, _P, _P, _P, _P, _I, _I, _I, _I, _I, _I, _I, _F, _F, _I, _P, _I, _I, _I, _I, _P, _P],
+    "tl_attention_generic": [_P, _I, _P, _I, _P, _P, _P, _P, _P, _I, _I, _I, _I, _I, _I, _I, _F, _F, _I, _P, _I, _I, _I, _I, _I, _P],
+    "tl_attention_generic_split": [_P, _I, _P, _I, _P, _P, _P, _P, _P, _I, _I, _I, _I, _I, _I, _I, _F, _F, _I, _P, _I, _I, _I, _I, _P, _I, _I, _P],
     "tl_embed_scaled": [_P, _P, _P, _I, _I, _F, _I, _P],
     "tl_layernorm": [_P, _P, _P, _F, _P, _P, _P, _P, _P, _I, _I, _F, _I, _I, _P],
     "tl_gelu_mul": [_P, _P, _I, _I, _I, _P],
     "tl_rope_norm_kv_write": [_P, _I, _I, _I, _I, _I, _P, _I, _I, _F, _P, _P, _P, _I, _I, _P],
     "tl_causal_conv": [_P, _I, _P, _P, _P, _I64, _P, _P, _P, _P, _I, _I, _I, _I, _I, _I, _I, _P],
     "tl_selective_scan": [_P, _P, _I, _P, _I, _I, _I, _P, _I, _P, _P, _P, _P, _I64, _P, _P, _P, _I, _I, _I, _I, _P, _P, _I, _P, _P, _P],
-    "tl_gated_delta": [_P, _I, _P, _I, _I, _I, _I, _P, _P, _P, _F, _P, _I64, _P, _P, _P, _I, _I, _I, _I, _I, _I, _P, _I, _P, _I, _I, _P, _I, _P],
+    "tl_gated_delta": [_P, _I, _P, _I, _I, _I, _I, _P, _P, _P, _F, _P, _I64, _P, _P, _P, _I, _I, _I, _I, _I, _I, _P, _I, _P, _I, _I, _P, _I, _F, _P],
     "tl_matrix_memory": [_P, _I, _I, _I, _I, _I, _I, _P, _P, _F, _P, _I, _I, _P, _F, _P, _I64, _P, _P, _P, _I, _I, _I, _I, _I, _P, _P, _I, _P],
-    "tl_router_topk": [_P, _I, _P, _I, _I, _I, _P, _P, _P],
+    "tl_router_topk": [_P, _I, _P, _I, _I, _I, _P, _P, _I, _I, _I, _F, _P],
+    "tl_streams_update": [_P, _I, _I64, _I, _I, _P, _I, _P, _P, _P, _P, _P, _P, _P, _P, _I, _P],
+    "tl_streams_open": [_P, _P, _I, _I64, _P],
+    "tl_maps_join": [_P, _I, _P, _I, _I, _I, _F, _F, _F, _I, _P],
     "tl_expert_glu_rows": [_P, _P, _P, _I, _P, _I, _I, _I, _I, _P],
     "tl_expert_down_rows": [_P, _P, _P, _I, _P, _I, _I, _I, _I, _P],
     "tl_expert_gather": [_P, _P, _I, _I, _I, _P, _P, _P, _P, _P, _I, _I, _P],

@@ -15,6 +15,8 @@ a module's own helpers and tables stay in the module.
                      rotation, query factor, mixed values), gates, packing for attention through a latent, logit cap
 ``routed_ops``       router (softmax scores, corrected choice), experts over the rows that chose them, bias with the
                      exact gelu, the norm behind a branch together with the norm before the next
+``stream_ops``       several residual streams with their weighted reads and writes, the norm without statistics,
+                     the join of differential attention's two maps
 ``sampling_ops``     the sampling kernel
 """
 
@@ -100,6 +102,7 @@ from .sequence_ops import (  # noqa: F401
     causal_conv,
     embed_scaled,
     gated_delta,
+    gated_linear,
     gelu_mul,
     layernorm,
     matrix_memory,
@@ -130,6 +133,12 @@ from .routed_ops import (  # noqa: F401
     post_norm_add_norm,
     router_topk,
     weighted_pair,
+)
+from .stream_ops import (  # noqa: F401
+    MAX_STREAMS,
+    maps_join,
+    streams_open,
+    streams_update,
 )
 from .sampling_ops import (  # noqa: F401
     philox_uniform,

@@ -15,22 +15,28 @@ from .base import F32, KernelError, _gpu, _ptr, _stream, check, core, dtype_code
 ROUTER_MAX_OUTPUTS = 512
 
 
-def router_topk(z: torch.Tensor, n_out: int, correction: torch.Tensor, top: int) -> Tuple[torch.Tensor, torch.Tensor]:
+def router_topk(z: torch.Tensor, n_out: int, correction: Optional[torch.Tensor], top: int, groups: int = 0, keep_groups: int = 0,
+                normalize: bool = False, scale: float = 1.0) -> Tuple[torch.Tensor, torch.Tensor]:
     """``z`` float32 [n, >= n_out]: the router's outputs in the first ``n_out`` columns.  ``s = softmax(z)``; the
     ``top`` outputs with the largest ``s + correction`` are chosen (of equal ones the lower index).  Returns
-    ``(ids int32 [n, top], weights float32 [n, top])``, the weights being the chosen outputs' ``s``."""
+    ``(ids int32 [n, top], weights float32 [n, top])``, the weights being the chosen outputs' ``s``.  ``correction``
+    None: the largest ``s``.  ``groups`` g > 0: the outputs form g equal groups of neighbours, a group's score is the
+    largest ``s`` in it, and only outputs of the ``keep_groups`` best groups can be chosen.  ``normalize``: the weights
+    are divided by their sum (+ 1e-20); ``scale`` then multiplies them."""
     _gpu(z, correction)
     if z.dim() != 2 or z.dtype != torch.float32 or z.stride(1) != 1 or z.shape[1] < n_out:
         raise KernelError(f"router_topk: z must be float32 [n, >= {n_out}] with contiguous rows")
-    if tuple(correction.shape) != (n_out,) or correction.dtype != torch.float32 or not correction.is_contiguous():
+    if correction is not None and (tuple(correction.shape) != (n_out,) or correction.dtype != torch.float32 or not correction.is_contiguous()):
         raise KernelError(f"router_topk: correction must be a float32 vector of {n_out} entries")
     if not 0 < top <= n_out:
         raise KernelError(f"router_topk: {top} choices among {n_out} outputs")
+    if groups and (groups < 0 or groups > 64 or n_out % groups or not 0 < keep_groups <= groups or keep_groups * (n_out // groups) < top):
+        raise KernelError(f"router_topk: {groups} groups of which {keep_groups} stay do not fit {n_out} outputs and {top} choices (at most 64 groups)")
     n = z.shape[0]
     ids = torch.empty((n, top), dtype=torch.int32, device=z.device)
     weights = torch.empty((n, top), dtype=torch.float32, device=z.device)
-    check(core().tl_router_topk(z.data_ptr(), z.stride(0), correction.data_ptr(), n, n_out, top, ids.data_ptr(), weights.data_ptr(),
-                                _stream()))
+    check(core().tl_router_topk(z.data_ptr(), z.stride(0), _ptr(correction), n, n_out, top, ids.data_ptr(), weights.data_ptr(),
+                                int(groups), int(keep_groups), 1 if normalize else 0, float(scale), _stream()))
     return ids, weights
 
 
@@ -146,7 +152,7 @@ def expert_combine(
     shared_gate: Optional[torch.Tensor] = None,
 ) -> torch.Tensor:
     """``out[t] = sum_j weights[t, j] * (y[pos[t, j]] if ids[t, j] < n_experts else x[t])``, plus
-    ``sigmoid(shared_gate[t]) * shared[t]``: the experts' results (rows in the order ``expert_gather`` gave them) back
+    ``sigmoid(shared_gate[t]) * shared[t]`` (``shared[t]`` as it is without a gate): the experts' results (rows in the order ``expert_gather`` gave them) back
     in the order of the tokens; ``y`` is 32-bit (``expert_down_rows``) or of x's dtype (matrix products over the
     gathered rows).  Returns [n, D] of x's dtype."""
     _gpu(y, pos, ids, weights, x, shared, shared_gate)
@@ -163,9 +169,9 @@ def expert_combine(
     if shared is not None:
         if tuple(shared.shape) != (n, D) or shared.dtype != x.dtype or not shared.is_contiguous():
             raise KernelError("expert_combine: the shared expert's result must be contiguous [n, D] of x's dtype")
-        if shared_gate is None or shared_gate.dtype != torch.float32 or shared_gate.numel() != n or shared_gate.dim() > 2:
+        if shared_gate is not None and (shared_gate.dtype != torch.float32 or shared_gate.numel() != n or shared_gate.dim() > 2):
             raise KernelError("expert_combine: the shared expert's gate must be float32, one number a token")
-        sg_stride = shared_gate.stride(0) if n > 1 else 1
+        sg_stride = shared_gate.stride(0) if (n > 1 and shared_gate is not None) else 1
     out = torch.empty((n, D), dtype=x.dtype, device=x.device)
     check(core().tl_expert_combine(y.data_ptr(), 1 if y.dtype == torch.float32 else 0, pos.data_ptr(), ids.data_ptr(), weights.data_ptr(), top, n_experts, x.data_ptr(),
                                    _ptr(shared), _ptr(shared_gate), sg_stride, out.data_ptr(), n, D, dtype_code(x.dtype), _stream()))

@@ -353,6 +353,58 @@ def gated_delta(
             dt_bias.data_ptr(), norm_weight.data_ptr(), float(eps), region, stride, qo_indptr.data_ptr(), slot_ids.data_ptr(),
             out.data_ptr(), n, n_seqs, H, G, dk, dv, o_raw.data_ptr(), dtype_code(qkv.dtype), gate_src.data_ptr(), gate_src.stride(0),
             1 if gate_act == "sigmoid" else 0, _ptr(channel_decay), channel_decay.stride(0) if channel_decay is not None else 0,
+            0.0, _stream(),
+        )
+    )
+    return out
+
+
+def gated_linear(
+    qkv: torch.Tensor,
+    decay_pre: torch.Tensor,
+    decay_bias: torch.Tensor,
+    decay_power: float,
+    gate: torch.Tensor,
+    gate_offset: int,
+    norm_weight: torch.Tensor,
+    eps: float,
+    state: torch.Tensor,
+    state_offset: int,
+    qo_indptr: torch.Tensor,
+    slot_ids: torch.Tensor,
+    n_heads: int,
+    head_dim: int,
+    v_head_dim: int,
+) -> torch.Tensor:
+    """Gated linear attention over each request's tokens, in 32-bit.  ``qkv`` [n, 2 H dk + H dv]: query heads | key
+    heads | value heads as projected.  Per head, with q times dk^-1/2 and a decay for every key channel
+    ``alpha = sigmoid(decay_pre[t, h, i] + decay_bias[h, i]) ** decay_power`` (``decay_pre`` float32 [n, H * dk]):
+    ``S <- diag(alpha) S + k v^T; o = S^T q``; then o over its root mean square, times ``norm_weight`` [dv], times
+    silu of the gate (H dv columns of ``gate`` from ``gate_offset``).  ``S`` lives at ``state_offset`` of the request's
+    state row, H * dv * dk floats.  Returns [n, H * dv].  The recurrence is the delta rule's kernel with its plain rule."""
+    _gpu(qkv, decay_pre, decay_bias, gate, norm_weight)
+    H, dk, dv = n_heads, head_dim, v_head_dim
+    n = qkv.shape[0]
+    if qkv.dim() != 2 or qkv.shape[1] != 2 * H * dk + H * dv or qkv.stride(1) != 1:
+        raise KernelError(f"gated_linear: qkv must be [n, {2 * H * dk + H * dv}] with contiguous rows")
+    if gate.dim() != 2 or gate.shape[0] != n or gate.stride(1) != 1 or gate.dtype != qkv.dtype or gate_offset < 0 or gate_offset + H * dv > gate.shape[1]:
+        raise KernelError("gated_linear: the gate must be a matrix of qkv's dtype with a row per token that holds H * dv columns from gate_offset")
+    if decay_pre.dim() != 2 or tuple(decay_pre.shape) != (n, H * dk) or decay_pre.dtype != torch.float32 or decay_pre.stride(1) != 1:
+        raise KernelError(f"gated_linear: decay_pre must be float32 [n, {H * dk}] with contiguous rows")
+    for v, size in ((decay_bias, H * dk), (norm_weight, dv)):
+        if tuple(v.shape) != (size,) or v.dtype != torch.float32 or not v.is_contiguous():
+            raise KernelError(f"gated_linear: a float32 vector of {size} entries expected, got {tuple(v.shape)} {v.dtype}")
+    if not decay_power > 0:
+        raise KernelError("gated_linear: the decay's power must be positive")
+    n_seqs = _step_rows(None, qo_indptr, slot_ids, n, state)
+    region, stride = state_region(state, state_offset, H * dv * dk)
+    out = torch.empty((n, H * dv), dtype=qkv.dtype, device=qkv.device)
+    o_raw = torch.empty((n, H * dv), dtype=torch.float32, device=qkv.device)
+    check(
+        core().tl_gated_delta(
+            qkv.data_ptr(), qkv.stride(0), None, 0, gate_offset, 0, 0, None, decay_bias.data_ptr(), norm_weight.data_ptr(), float(eps),
+            region, stride, qo_indptr.data_ptr(), slot_ids.data_ptr(), out.data_ptr(), n, n_seqs, H, H, dk, dv, o_raw.data_ptr(),
+            dtype_code(qkv.dtype), gate.data_ptr(), gate.stride(0), 0, decay_pre.data_ptr(), decay_pre.stride(0), float(decay_power),
             _stream(),
         )
     )

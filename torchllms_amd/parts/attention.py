@@ -10,7 +10,8 @@ import torch
 from ..config.spec import PartSpec
 from ..kernels import ops
 from ..kernels.attention import paged_attention
-from .base import MIXERS, POSITIONS, KVNeed, Mixer, ParamSpec
+from .base import MIXERS, POSITIONS, KVNeed, Mixer, ParamSpec, StateNeed
+from .positions import step_table
 
 
 #: (heads, kv heads, head size) whose fall to the plain attention kernel has been reported
@@ -45,6 +46,9 @@ class Attention(Mixer):
 
     ``values_from_keys``: there is no value projection; a token's values are its keys as projected, before the
     rotation (the key rows of the fused projection stand in it a second time as value rows).
+
+    ``keep_first`` n > 0 (with a window): a query also sees the first n positions of its request, at their true
+    positions; their pages are never given back.
     """
 
     #: every launch is fixed by the step's shape: a decode step may be recorded in a HIP graph
@@ -75,8 +79,12 @@ class Attention(Mixer):
         value_mix_key: str = "values",
         out_gate: Optional[str] = None,
         values_from_keys: bool = False,
+        keep_first: int = 0,
     ):
         self.values_from_keys = bool(values_from_keys)
+        self.keep_first = int(keep_first)
+        if self.keep_first < 0:
+            raise ValueError("attention: keep_first must not be negative")
         if self.values_from_keys and (shares_kv or (v_head_dim and v_head_dim != head_dim) or qkv_bias):
             raise ValueError("attention: values that are the keys have the keys' head size, no bias, and a cache of their own")
         if num_heads % num_kv_heads:
@@ -194,7 +202,8 @@ class Attention(Mixer):
         if self.shares_kv:
             return None
         return KVNeed(num_kv_heads=self.num_kv_heads, head_dim=self.head_dim, window=self.window, page_size=self.kv_page_size,
-                      v_head_dim=self.v_head_dim if self.v_head_dim != self.head_dim else None)
+                      v_head_dim=self.v_head_dim if self.v_head_dim != self.head_dim else None,
+                      keep_first=self.keep_first if self.window > 0 else 0)
 
     def bind(self, tensors: Dict[str, torch.Tensor]) -> None:
         names = ["wq"] if self.shares_kv else ["wq", "wk", "wk" if self.values_from_keys else "wv"]
@@ -224,10 +233,7 @@ class Attention(Mixer):
         # whose position encoding has the same frequencies
         table = None
         if rot is not None and rot.rotary_dim > 0:
-            key = ("rope_table", rot.inv_freq.data_ptr())
-            table = ctx.scratch.get(key)
-            if table is None:
-                table = ctx.scratch[key] = ops.rope_table(ctx.positions, rot.inv_freq)
+            table = step_table(rot, ctx)
         if self.prepared:
             return self._forward_prepared(x, ctx, cache, n_kv_in_row, rot, table, store)
         if self.extended:
@@ -251,7 +257,7 @@ class Attention(Mixer):
         )
         attn = paged_attention(
             qkv, self.num_heads, self.num_kv_heads, self.head_dim, cache.k_pages, cache.v_pages,
-            ctx, g, self.window, self.softmax_scale,
+            ctx, g, self.window, self.softmax_scale, keep_first=self.keep_first,
         )
         return ops.linear_to_sum(attn, self.wo, may_wait=True)
 
@@ -270,6 +276,7 @@ class Attention(Mixer):
         attn = paged_attention(
             qkv, self.num_heads, self.num_kv_heads, self.head_dim, cache.k_pages, cache.v_pages, ctx, g, self.window,
             self.softmax_scale, softcap=self.softcap, chunk=self.chunk, sinks=self.sinks, v_head_dim=self.v_head_dim,
+            keep_first=self.keep_first,
         )
         return ops.linear_to_sum(attn, self.wo, may_wait=True)
 
@@ -299,9 +306,142 @@ class Attention(Mixer):
             ctx.scratch[("value_mix", self.value_mix_key)] = rows[:, v_at : v_at + n_kv_in_row * dv]
         attn = paged_attention(
             rows, H, self.num_kv_heads, dk, cache.k_pages, cache.v_pages, ctx, g, self.window, self.softmax_scale,
-            softcap=self.softcap, chunk=self.chunk, sinks=self.sinks, v_head_dim=dv,
+            softcap=self.softcap, chunk=self.chunk, sinks=self.sinks, v_head_dim=dv, keep_first=self.keep_first,
         )
         if self.out_gate is not None:
             gate_at = v_at + n_kv_in_row * dv
             ops.sigmoid_gate_(attn, rows[:, gate_at : gate_at + self.gate_rows], per=1 if self.out_gate == "channel" else dv)
         return ops.linear_to_sum(attn, self.wo, may_wait=True)
+
+
+def covering_window(masks) -> tuple:
+    """``(window, keep_first)`` of the pages that serve every one of ``masks`` (pairs ``(window, keep_first)``, window 0:
+    every key stays): what the layer that owns keys and values asks of the cache when other layers read them too."""
+    masks = list(masks)
+    if any(w <= 0 for w, _ in masks):
+        return 0, 0
+    return max(w for w, _ in masks), max(k for _, k in masks)
+
+
+@MIXERS.register("differential_attention")
+class DifferentialAttention(Mixer):
+    """Differential attention: every head has two softmax maps over the same values, each with queries and keys of its
+    own (``head_dim`` channels a map), and the head's output is ``a_1 - lambda a_2`` divided by its root mean square
+    over ``v_head_dim`` (eps under the root, no weight), times ``1 - diff``; ``lambda = exp(lq1 . lk1) - exp(lq2 . lk2) +
+    diff`` is one number of the layer.  Query head h reads key/value head ``h // (num_heads / num_kv_heads)``.
+
+    Tensors ``q`` [H * 2 * d, hidden], ``k`` [G * 2 * d, hidden] (head by head as [map 1, map 2]), ``v`` [G * dv, hidden],
+    ``o``, ``lq1``, ``lk1``, ``lq2``, ``lk2`` [d]; ``conv_taps`` K > 0: a causal convolution over K taps on every channel
+    of q, k and v right behind the projection (tensors ``q.conv`` ... [channels, K], no bias, no activation), whose last
+    K - 1 inputs per request are state.  Then the rotation of every map (``position``), the cache write, causal softmax
+    attention inside ``window`` (0: none) plus the first ``keep_first`` positions.
+
+    In the cache the two maps are heads of their own: keys lie as ``2 G`` heads, map 1 of all kv heads and then map 2,
+    so that the grouped mapping of query heads to key heads holds for each map, and the values as ``G`` heads that
+    both maps read (``KVNeed.num_v_heads``).  The weights are put into that order when they arrive.  ``shares_kv``: no
+    k and v tensors; the run reads the pages of the run that the execution order names, with its own queries, their
+    convolution and its own mask; ``cache_window`` / ``cache_keep_first``: what the pages must serve when other layers
+    read them too (default: this layer's own mask)."""
+
+    graph_safe = True
+
+    def __init__(self, hidden_size: int, num_heads: int, num_kv_heads: int, head_dim: int, v_head_dim: int, softmax_scale: float,
+                 diff: float, norm_eps: float, window: int, position: PartSpec, keep_first: int = 0, conv_taps: int = 0,
+                 shares_kv: bool = False, kv_page_size: Optional[int] = None, cache_window: Optional[int] = None,
+                 cache_keep_first: Optional[int] = None):
+        if num_heads % num_kv_heads:
+            raise ValueError(f"differential attention: {num_heads} heads are not a multiple of {num_kv_heads} kv heads")
+        if window < 0 or keep_first < 0 or conv_taps < 0:
+            raise ValueError("differential attention: window, keep_first and conv_taps must not be negative")
+        self.hidden_size, self.H, self.G, self.d, self.dv = hidden_size, num_heads, num_kv_heads, head_dim, v_head_dim
+        self.softmax_scale, self.diff, self.norm_eps = float(softmax_scale), float(diff), float(norm_eps)
+        self.window, self.keep_first, self.taps = int(window), int(keep_first), int(conv_taps)
+        self.shares_kv, self.kv_page_size = bool(shares_kv), kv_page_size
+        self.cache_window = self.window if cache_window is None else int(cache_window)
+        self.cache_keep_first = self.keep_first if cache_keep_first is None else int(cache_keep_first)
+        self.position = POSITIONS.build(position)
+        self.wqkv = self.wo = self.conv_w = None
+        self.lam = 0.0
+
+    @property
+    def q_cols(self) -> int:
+        return 2 * self.H * self.d
+
+    @property
+    def channels(self) -> int:
+        """Columns of the fused projection (and channels of the convolution)."""
+        return self.q_cols + (0 if self.shares_kv else 2 * self.G * self.d + self.G * self.dv)
+
+    def param_specs(self) -> Dict[str, ParamSpec]:
+        D, d = self.hidden_size, self.d
+        sizes = {"q": self.q_cols} if self.shares_kv else {"q": self.q_cols, "k": 2 * self.G * d, "v": self.G * self.dv}
+        specs = {name: ParamSpec((rows, D)) for name, rows in sizes.items()}
+        if self.taps > 0:
+            specs.update({f"{name}.conv": ParamSpec((rows, self.taps), init="conv") for name, rows in sizes.items()})
+        for name in ("lq1", "lk1", "lq2", "lk2"):
+            specs[name] = ParamSpec((d,), kind="vector", init="normal")
+        specs["o"] = ParamSpec((D, self.H * self.dv))
+        return specs
+
+    def check_sizes(self, dtype: torch.dtype) -> None:
+        if not 0 < self.dv <= ops.ATTENTION_MAX_HEAD_DIM or not 0 < self.d <= min(ops.ATTENTION_MAX_KEY_DIM, ops.HEAD_PREPARE_MAX_DIM):
+            raise ValueError(f"differential attention: heads of {self.d} channels with values of {self.dv}; the kernels take "
+                             f"{min(ops.ATTENTION_MAX_KEY_DIM, ops.HEAD_PREPARE_MAX_DIM)} and {ops.ATTENTION_MAX_HEAD_DIM}")
+        if self.taps > 64:
+            raise ValueError(f"differential attention: a convolution over {self.taps} taps; the kernel takes up to 64")
+        rotated = getattr(self.position, "rotary_dim", 0)
+        if rotated % 2 or rotated > self.d:
+            raise ValueError(f"differential attention: {rotated} rotated channels of a map of {self.d}")
+
+    def cache_need(self):
+        needs = {}
+        if not self.shares_kv:
+            needs["kv"] = KVNeed(num_kv_heads=2 * self.G, head_dim=self.d, window=self.cache_window, page_size=self.kv_page_size,
+                                 v_head_dim=self.dv, keep_first=self.cache_keep_first if self.cache_window > 0 else 0, num_v_heads=self.G)
+        if self.taps > 0:  # (one tap has no history; the row is never empty, so that there is a tensor to point at)
+            needs["conv"] = StateNeed(shape=(max((self.taps - 1) * self.channels, 1),), dtype="float32")
+        return needs
+
+    def _maps_first(self, t: torch.Tensor, heads: int) -> torch.Tensor:
+        """Rows stored head by head as [map 1, map 2] -> map 1 of all heads, then map 2."""
+        return t.reshape(heads, 2, self.d, *t.shape[1:]).transpose(0, 1).reshape(t.shape).contiguous()
+
+    def bind(self, tensors: Dict[str, torch.Tensor]) -> None:
+        parts = [("q", self.H)] if self.shares_kv else [("q", self.H), ("k", self.G), ("v", 0)]
+        ordered = lambda name, heads, suffix="": (self._maps_first(tensors[name + suffix], heads) if heads else tensors[name + suffix])  # noqa: E731
+        self.wqkv = torch.cat([ordered(n, h) for n, h in parts], dim=0).contiguous()
+        if self.taps > 0:
+            self.conv_w = torch.cat([ordered(n, h, ".conv") for n, h in parts], dim=0).float().t().contiguous()  # [taps, channels]
+        self.wo = tensors["o"].contiguous()
+        f = {n: tensors[n].float() for n in ("lq1", "lk1", "lq2", "lk2")}
+        self.lam = float(torch.exp((f["lq1"] * f["lk1"]).sum()) - torch.exp((f["lq2"] * f["lk2"]).sum())) + self.diff
+        self.position.to(self.wo.device)
+
+    def linear_weights(self):
+        return [self.wqkv, (self.wo, "sum")]
+
+    def forward(self, x, ctx, cache):
+        H, G, d, dv = self.H, self.G, self.d, self.dv
+        kv = cache["kv"]
+        g = kv.group
+        store = kv.writes and not self.shares_kv
+        rows = ops.linear(ops.resolved(x), self.wqkv)
+        if self.taps > 0:
+            rows = ops.causal_conv(rows, self.conv_w, None, cache["conv"].tensor, 0, ctx.token_seq, ctx.qo_indptr, ctx.slot_ids, silu=False)
+        rot = self.position.rotary_args()
+        table = step_table(rot, ctx) if rot is not None and rot.rotary_dim > 0 else None
+        n_k = 0 if self.shares_kv else 2 * G
+        # every map is a head of its own for the rotation and in the pages
+        ops.head_prepare(
+            rows, 2 * H, n_k, d, 0, cos_sin=table, rot_offset=0, rot_dims=rot.rotary_dim if table is not None else 0,
+            pairing=rot.pairing if rot else 0, k_pages=kv.k_pages if store else None,
+            slot_mapping=ctx.slot_mappings[g] if store else None, page_size=kv.page_size if store else 0,
+        )
+        if store:
+            # the values go to their pages as they are (to the kernel they are heads without norm or rotation)
+            ops.head_prepare(rows[:, (2 * H + n_k) * d :], 0, G, dv, 0, k_pages=kv.v_pages, slot_mapping=ctx.slot_mappings[g],
+                             page_size=kv.page_size)
+        maps = paged_attention(rows, 2 * H, 2 * G, d, kv.k_pages, kv.v_pages, ctx, g, self.window, self.softmax_scale,
+                               v_head_dim=dv, keep_first=self.keep_first, value_heads=G)
+        out = ops.maps_join(maps, H, dv, self.lam, self.norm_eps, 1.0 - self.diff)
+        return ops.linear_to_sum(out, self.wo, may_wait=True)

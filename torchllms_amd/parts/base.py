@@ -35,7 +35,7 @@ class ParamSpec:
     tensor stored in 32-bit stays in 32-bit), "int" (an integer table, kept as int32).
     ``init``: how the random-weights mode fills it: "normal" N(0, 0.02), "ones", "zeros", "conv" and "wide" (N(0, 0.5):
     the taps of a short convolution, a projection from very few inputs), "fraction" (uniform between 0.25 and 0.75: a
-    mixing factor).
+    mixing factor), "near_identity" (a small square matrix: the identity and a little of everything).
     """
 
     shape: Tuple[int, ...]
@@ -55,6 +55,8 @@ class KVNeed:
     ``values_in_keys``: a token's value is the first ``v_head_dim`` channels of its key row (attention through a
     latent: the latent is the value and, with the rotated part behind it, the key), so no value pages are kept and
     a mixer's ``v_pages`` is its ``k_pages``.
+    ``keep_first`` n > 0 (with a window): the first n positions of a request stay visible, so the pages that hold
+    them are never given back.  ``num_v_heads``: heads of the value pages when they are fewer than the key pages'.
     """
 
     num_kv_heads: int
@@ -64,6 +66,8 @@ class KVNeed:
     dtype: Optional[str] = None
     v_head_dim: Optional[int] = None
     values_in_keys: bool = False
+    keep_first: int = 0
+    num_v_heads: Optional[int] = None
 
 
 @dataclass(frozen=True)
@@ -173,7 +177,9 @@ class FeedForward(Part):
 
 class Mixer(Part):
     def cache_need(self):
-        """``KVNeed``, ``StateNeed`` or None."""
+        """``KVNeed``, ``StateNeed`` or None; or a dict name -> need for a mixer that keeps several things (pages and a
+        state row, say): its ``forward`` is then handed a dict name -> view.  In a run that borrows another run's
+        cache, the pages (``KVNeed``) come from that run and the state stays the run's own."""
         return None
 
     def forward(self, x: torch.Tensor, ctx, cache) -> torch.Tensor:

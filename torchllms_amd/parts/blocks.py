@@ -2,8 +2,12 @@
 
 from __future__ import annotations
 
+from typing import Dict, Optional
+
+import torch
+
 from ..kernels import ops
-from .base import BLOCKS, Block
+from .base import BLOCKS, Block, ParamSpec
 
 
 @BLOCKS.register("pre_norm")
@@ -211,3 +215,118 @@ class SandwichPairMixerBlock(_SandwichPair):
     """The same layer without a feed-forward."""
 
     SLOTS = {"norm1": "norm", "left": "mixer", "right": "mixer", "norm1b": "norm"}
+
+
+class _Hyper(Block):
+    """Layers over several residual streams (hyper-connections).  Instead of one stream there are ``streams`` 32-bit
+    copies ``x_1 .. x_S`` (all equal to the embedding's rows when the first such layer opens them).  Sublayer q
+    (1: the mixer, 2: the feed-forward) reads ``u = sum_s in_q[s] x_s``, works on ``norm_q(u)``, and its result y goes
+    back into all streams at once, ``x_r <- sum_s mix_q[s, r] x_s + out_q[r] y``: the tensors ``hc<q>.in`` [S],
+    ``hc<q>.out`` [S] and ``hc<q>.mix`` [S, S] (indexed [from, to]) are the arrangement's own.  A sublayer's write, the
+    next sublayer's read and its norm are one kernel over the rows (also across layers, when the next layer is of
+    this kind: ``expects``).  The norms take several streams (``dynamic_tanh``); whoever reads the model's last
+    streams (the final norm) takes their plain sum."""
+
+    graph_safe = True
+    _ROWS = "hyper_rows"  # in ctx.scratch: (the streams the rows were made from, the norm that made them, the rows)
+
+    def __init__(self, parts, streams: int):
+        super().__init__(parts)
+        if not isinstance(streams, int) or not 0 < streams <= ops.MAX_STREAMS:
+            raise ValueError(f"hyper-connections: {streams!r} streams (1 to {ops.MAX_STREAMS})")
+        self.streams = streams
+        self.has_mlp = "mlp" in self.parts
+        self.hc: Dict[str, torch.Tensor] = {}
+        self.next_block: Optional["_Hyper"] = None
+
+    def own_specs(self) -> Dict[str, ParamSpec]:
+        S, specs = self.streams, {}
+        for q in ("hc1", "hc2") if self.has_mlp else ("hc1",):
+            specs[f"{q}.in"] = ParamSpec((S,), kind="matrix", init="fraction")
+            specs[f"{q}.out"] = ParamSpec((S,), kind="matrix", init="fraction")
+            specs[f"{q}.mix"] = ParamSpec((S, S), kind="matrix", init="near_identity")
+        return specs
+
+    def param_specs(self) -> Dict[str, ParamSpec]:
+        specs = super().param_specs()
+        specs.update(self.own_specs())
+        return specs
+
+    def bind(self, tensors) -> None:
+        super().bind(tensors)
+        self.hc = {name: tensors[name].float().contiguous() for name in self.own_specs()}
+
+    def expects(self, following) -> None:
+        self.next_block = following if isinstance(following, _Hyper) and following.streams == self.streams else None
+
+    def mix_branch(self, y, ctx, cache):
+        raise NotImplementedError
+
+    def forward(self, h, delta, ctx, cache):
+        if delta is not None:
+            if h.dim() == 3:
+                raise ValueError("hyper-connections: a sum that is not applied yet cannot be added to several streams")
+            h = h + ops.resolved(delta).float()
+        if h.dim() == 2:
+            h = ops.streams_open(h if h.dtype == torch.float32 else h.float(), self.streams)
+        kept = ctx.scratch.get(self._ROWS)
+        if kept is not None and kept[0] is h and kept[1] is self.norm1:
+            y = kept[2]
+        else:
+            y = self.norm1.read(h, self.hc["hc1.in"])
+        a = ops.resolved(self.mix_branch(y, ctx, cache))
+        last, mix, out = a, self.hc["hc1.mix"], self.hc["hc1.out"]
+        if self.has_mlp:
+            y = self.norm2.read(h, self.hc["hc2.in"], branch=a, mix=mix, out_weights=out)
+            last, mix, out = ops.resolved(self.mlp.forward(y, ctx)), self.hc["hc2.mix"], self.hc["hc2.out"]
+        nxt = self.next_block
+        if nxt is not None:
+            y = nxt.norm1.read(h, nxt.hc["hc1.in"], branch=last, mix=mix, out_weights=out)
+            ctx.scratch[self._ROWS] = (h, nxt.norm1, y)
+        else:
+            ops.streams_update(h, branch=last, mix=mix, out_weights=out)
+        return h, None
+
+
+@BLOCKS.register("hyper")
+class HyperBlock(_Hyper):
+    """A mixer and a feed-forward over several streams."""
+
+    SLOTS = {"norm1": "norm", "mix": "mixer", "norm2": "norm", "mlp": "feed_forward"}
+
+    def mix_branch(self, y, ctx, cache):
+        return self.mix.forward(y, ctx, cache["mix"])
+
+
+@BLOCKS.register("hyper_mixer")
+class HyperMixerBlock(_Hyper):
+    """The same layer without a feed-forward."""
+
+    SLOTS = {"norm1": "norm", "mix": "mixer"}
+
+    def mix_branch(self, y, ctx, cache):
+        return self.mix.forward(y, ctx, cache["mix"])
+
+
+class _HyperPair(_Hyper):
+    """Two mixers side by side that read the same normed rows; the mixer's result is
+    ``left_scale * left(h) + right_scale * right(h)``.  Each keeps a cache entry of its own."""
+
+    def __init__(self, parts, streams: int, left_scale: float = 1.0, right_scale: float = 1.0):
+        super().__init__(parts, streams)
+        self.left_scale, self.right_scale = float(left_scale), float(right_scale)
+
+    def mix_branch(self, y, ctx, cache):
+        a = ops.resolved(self.left.forward(y, ctx, cache["left"]))
+        b = ops.resolved(self.right.forward(y, ctx, cache["right"]))
+        return ops.weighted_pair(a, self.left_scale, b, self.right_scale)
+
+
+@BLOCKS.register("hyper_pair")
+class HyperPairBlock(_HyperPair):
+    SLOTS = {"norm1": "norm", "left": "mixer", "right": "mixer", "norm2": "norm", "mlp": "feed_forward"}
+
+
+@BLOCKS.register("hyper_pair_mixer")
+class HyperPairMixerBlock(_HyperPair):
+    SLOTS = {"norm1": "norm", "left": "mixer", "right": "mixer"}

@@ -77,7 +77,11 @@ class RoutedExperts(FeedForward):
     the last ``num_identity`` stand for experts that hand their input through.  Scores ``s = softmax(z)`` over all
     outputs; the ``top`` outputs with the largest ``s + correction`` are chosen, and the result is the sum of the
     chosen experts' outputs times their ``s`` (not renormalised).  ``shared_size`` f > 0: an expert of that width runs
-    for every token and is added times ``sigmoid(W_sg x)``, one number a token.
+    for every token and is added times ``sigmoid(W_sg x)``, one number a token (``shared_gate`` False: as it is).
+    ``correction`` False: there is no correction, the largest scores are chosen.  ``groups`` g > 0 with ``keep_groups``:
+    the experts form g equal groups of neighbours, a group's score is the largest score in it, and only experts of
+    the best ``keep_groups`` groups can be chosen.  ``normalize``: the chosen scores are divided by their sum
+    (+ 1e-20); ``route_scale`` then multiplies them.
 
     A token's result depends on nothing but the token.  The (token, choice) pairs of a step are put in the order of
     their experts on the device, and a kernel walks every expert's rows with the expert's weights read once for eight
@@ -92,19 +96,29 @@ class RoutedExperts(FeedForward):
     #: (token, choice) pairs of a bfloat16 step with prompts from which on the experts run as matrix products
     GROUPED_FROM = 512
 
-    def __init__(self, hidden_size: int, expert_size: int, num_experts: int, top: int, num_identity: int = 0, shared_size: int = 0):
+    def __init__(self, hidden_size: int, expert_size: int, num_experts: int, top: int, num_identity: int = 0, shared_size: int = 0,
+                 shared_gate: bool = True, correction: bool = True, groups: int = 0, keep_groups: int = 0, normalize: bool = False,
+                 route_scale: float = 1.0):
         for name, v in (("expert_size", expert_size), ("num_experts", num_experts), ("top", top)):
             if not isinstance(v, int) or v <= 0:
                 raise ValueError(f"routed: {name} must be a positive integer, got {v!r}")
         if num_identity < 0 or shared_size < 0 or top > num_experts + num_identity:
             raise ValueError(f"routed: {top} choices among {num_experts} + {num_identity} outputs; sizes must not be negative")
         self.hidden_size, self.F, self.E, self.I, self.top, self.shared = hidden_size, expert_size, num_experts, num_identity, top, shared_size
+        self.shared_gate, self.has_correction = bool(shared_gate) and shared_size > 0, bool(correction)
+        self.groups, self.keep_groups, self.normalize, self.route_scale = int(groups or 0), int(keep_groups or 0), bool(normalize), float(route_scale)
+        n_out = num_experts + num_identity
+        if self.groups and (self.groups < 0 or n_out % self.groups or not 0 < self.keep_groups <= self.groups
+                            or self.keep_groups * (n_out // self.groups) < top):
+            raise ValueError(f"routed: {self.groups} groups of which {self.keep_groups} stay do not fit {n_out} outputs and {top} choices")
         self.w_router = self.correction = self.w_gu = self.w_down = self.shared_w13 = self.shared_w2 = None
         self._rows_in_order: Dict[int, torch.Tensor] = {}
 
     def param_specs(self) -> Dict[str, ParamSpec]:
         d, f, n = self.hidden_size, self.F, self.E + self.I
-        specs = {"router.weight": ParamSpec((n, d), init="wide"), "correction": ParamSpec((n,), init="zeros")}
+        specs = {"router.weight": ParamSpec((n, d), init="wide")}
+        if self.has_correction:
+            specs["correction"] = ParamSpec((n,), init="zeros")
         for e in range(self.E):
             specs[f"experts.{e}.w1.weight"] = ParamSpec((f, d))
             specs[f"experts.{e}.w3.weight"] = ParamSpec((f, d))
@@ -113,10 +127,13 @@ class RoutedExperts(FeedForward):
             specs["shared.w1.weight"] = ParamSpec((self.shared, d))
             specs["shared.w3.weight"] = ParamSpec((self.shared, d))
             specs["shared.w2.weight"] = ParamSpec((d, self.shared))
-            specs["shared.gate.weight"] = ParamSpec((1, d))
+            if self.shared_gate:
+                specs["shared.gate.weight"] = ParamSpec((1, d))
         return specs
 
     def check_sizes(self, dtype: torch.dtype) -> None:
+        if self.groups > 64:
+            raise ValueError(f"routed: {self.groups} groups of experts; the kernel takes up to 64")
         if self.E + self.I > ops.ROUTER_MAX_OUTPUTS:
             raise ValueError(f"routed: a router of {self.E + self.I} outputs; the kernel takes up to {ops.ROUTER_MAX_OUTPUTS}")
         lds = ops.device_facts()[1]
@@ -125,9 +142,9 @@ class RoutedExperts(FeedForward):
 
     def bind(self, tensors: Dict[str, torch.Tensor]) -> None:
         # the router's matrix, and under it the shared expert's gate: one product with 32-bit results
-        rows = [tensors["router.weight"]] + ([tensors["shared.gate.weight"]] if self.shared else [])
+        rows = [tensors["router.weight"]] + ([tensors["shared.gate.weight"]] if self.shared_gate else [])
         self.w_router = torch.cat(rows, dim=0).contiguous()
-        self.correction = tensors["correction"].float().contiguous()
+        self.correction = tensors["correction"].float().contiguous() if self.has_correction else None
         self.w_gu = torch.stack([torch.cat([tensors[f"experts.{e}.w1.weight"], tensors[f"experts.{e}.w3.weight"]], dim=0)
                                  for e in range(self.E)]).contiguous()
         self.w_down = torch.stack([tensors[f"experts.{e}.w2.weight"] for e in range(self.E)]).contiguous()
@@ -149,11 +166,12 @@ class RoutedExperts(FeedForward):
         x = ops.resolved(x)
         n_out = self.E + self.I
         z = ops.linear(x, self.w_router, out_dtype=torch.float32)
-        ids, weights = ops.router_topk(z, n_out, self.correction, self.top)
+        ids, weights = ops.router_topk(z, n_out, self.correction, self.top, groups=self.groups, keep_groups=self.keep_groups,
+                                       normalize=self.normalize, scale=self.route_scale)
         shared = gate = None
         if self.shared:
             shared = ops.linear(ops.linear_glu(x, self.shared_w13), self.shared_w2)
-            gate = z[:, n_out]
+            gate = z[:, n_out] if self.shared_gate else None
         pairs = x.shape[0] * self.top
         if x.dtype == torch.bfloat16 and pairs <= ops.PAIR_PRODUCTS_MOST and self.hidden_size % 8 == 0 and self.F % 8 == 0:
             # a decode step of one or two requests: every pair by the dense layers' weight-streaming products

@@ -10,6 +10,7 @@ from ..config.spec import PartSpec
 from ..kernels import ops
 from ..kernels.attention import paged_attention
 from .base import MIXERS, POSITIONS, KVNeed, Mixer, ParamSpec
+from .positions import step_table
 
 
 @MIXERS.register("latent_attention")
@@ -36,13 +37,14 @@ class LatentAttention(Mixer):
         head_dim: int,
         rot_dim: int,
         v_head_dim: int,
-        q_rank: int,
+        q_rank: Optional[int],
         kv_rank: int,
         softmax_scale: float,
         norm_eps: float,
         position: PartSpec,
         head_gate: bool = False,
         kv_page_size: Optional[int] = None,
+        window: int = 0,
     ):
         if rot_dim < 0 or rot_dim % 2:
             raise ValueError(f"latent attention: {rot_dim} rotated channels (even, not negative)")
@@ -51,7 +53,10 @@ class LatentAttention(Mixer):
         self.head_dim = head_dim
         self.rot_dim = rot_dim
         self.v_head_dim = v_head_dim
-        self.q_rank = q_rank
+        self.q_rank = int(q_rank) if q_rank else 0  # 0: the queries are projected from the layer's input directly (tensor ``q``)
+        self.window = int(window)
+        if self.window < 0:
+            raise ValueError("latent attention: window must not be negative")
         self.kv_rank = kv_rank
         self.softmax_scale = float(softmax_scale)
         self.norm_eps = float(norm_eps)
@@ -74,15 +79,17 @@ class LatentAttention(Mixer):
     def param_specs(self) -> Dict[str, ParamSpec]:
         H, d, r, dv = self.num_heads, self.head_dim, self.rot_dim, self.v_head_dim
         specs = {
-            "dq.weight": ParamSpec((self.q_rank, self.hidden_size)),
-            "dq_norm.weight": ParamSpec((self.q_rank,), kind="vector", init="ones"),
-            "uq.weight": ParamSpec((H * (d + r), self.q_rank)),
             "dkv.weight": ParamSpec((self.kv_rank + r, self.hidden_size)),
             "dkv_norm.weight": ParamSpec((self.kv_rank,), kind="vector", init="ones"),
             "uk.weight": ParamSpec((H * d, self.kv_rank)),
             "uv.weight": ParamSpec((H * dv, self.kv_rank)),
             "wo.weight": ParamSpec((self.hidden_size, H * dv)),
         }
+        if self.q_rank:
+            specs.update({"dq.weight": ParamSpec((self.q_rank, self.hidden_size)), "dq_norm.weight": ParamSpec((self.q_rank,), kind="vector", init="ones"),
+                          "uq.weight": ParamSpec((H * (d + r), self.q_rank))})
+        else:
+            specs["q.weight"] = ParamSpec((H * (d + r), self.hidden_size))
         if self.head_gate:
             specs["wg.weight"] = ParamSpec((H, self.hidden_size))
         return specs
@@ -97,23 +104,25 @@ class LatentAttention(Mixer):
             raise ValueError("latent attention: the position encoding must rotate exactly the rotated part")
 
     def cache_need(self):
-        return KVNeed(num_kv_heads=1, head_dim=self.key_dim, window=0, page_size=self.kv_page_size, v_head_dim=self.kv_rank,
+        return KVNeed(num_kv_heads=1, head_dim=self.key_dim, window=self.window, page_size=self.kv_page_size, v_head_dim=self.kv_rank,
                       values_in_keys=True)
 
     def bind(self, tensors: Dict[str, torch.Tensor]) -> None:
         H, d, dv = self.num_heads, self.head_dim, self.v_head_dim
-        down = [tensors["dq.weight"], tensors["dkv.weight"]] + ([tensors["wg.weight"]] if self.head_gate else [])
+        # one product for [query latent, or the queries themselves | latent | shared rotated key part | gates]
+        first = tensors["dq.weight"] if self.q_rank else tensors["q.weight"]
+        down = [first, tensors["dkv.weight"]] + ([tensors["wg.weight"]] if self.head_gate else [])
         self.w_down = torch.cat(down, dim=0).contiguous()
-        self.w_uq = tensors["uq.weight"].contiguous()
+        self.w_uq = tensors["uq.weight"].contiguous() if self.q_rank else None
         self.w_uk_t = tensors["uk.weight"].reshape(H, d, self.kv_rank).transpose(1, 2).contiguous()
         self.w_uv = tensors["uv.weight"].reshape(H, dv, self.kv_rank).contiguous()
         self.wo = tensors["wo.weight"].contiguous()
-        self.q_norm = tensors["dq_norm.weight"].float().contiguous()
+        self.q_norm = tensors["dq_norm.weight"].float().contiguous() if self.q_rank else None
         self.kv_norm = tensors["dkv_norm.weight"].float().contiguous()
         self.position.to(self.wo.device)
 
     def linear_weights(self):
-        return [self.w_down, self.w_uq, (self.wo, "sum")]
+        return [self.w_down, self.w_uq, (self.wo, "sum")]  # (a None is skipped)
 
     def _per_head(self, x: torch.Tensor, w: torch.Tensor) -> torch.Tensor:
         """``out[h] = x[:, h, :] @ w[h].T`` as [H, n, rows of w[h]]: x a view [n, H, k] whose rows may lie apart."""
@@ -139,13 +148,13 @@ class LatentAttention(Mixer):
             outs = []
             for h0 in range(0, H, per_call):
                 hg = min(per_call, H - h0)
-                outs.append(paged_attention(queries[:, h0 * kd : (h0 + hg) * kd], hg, 1, kd, cache.k_pages, cache.v_pages, ctx, g, 0,
+                outs.append(paged_attention(queries[:, h0 * kd : (h0 + hg) * kd], hg, 1, kd, cache.k_pages, cache.v_pages, ctx, g, self.window,
                                             self.softmax_scale).view(n, hg, kd)[:, :, :R])
             return outs[0] if len(outs) == 1 else torch.cat(outs, dim=1)
         # the plain kernel reads the values out of the key rows; a latent wider than its values is mixed in pieces
         piece = ops.ATTENTION_MAX_HEAD_DIM
         parts = [
-            paged_attention(queries, H, 1, kd, cache.k_pages, cache.v_pages, ctx, g, 0, self.softmax_scale,
+            paged_attention(queries, H, 1, kd, cache.k_pages, cache.v_pages, ctx, g, self.window, self.softmax_scale,
                             v_head_dim=min(piece, R - at), values_in_keys=True, value_offset=at).view(n, H, -1)
             for at in range(0, R, piece)
         ]
@@ -157,28 +166,29 @@ class LatentAttention(Mixer):
         rot = self.position.rotary_args()
         table = None
         if r > 0:
-            key = ("rope_table", rot.inv_freq.data_ptr())
-            table = ctx.scratch.get(key)
-            if table is None:
-                table = ctx.scratch[key] = ops.rope_table(ctx.positions, rot.inv_freq)
+            table = step_table(rot, ctx)
         pairing = rot.pairing if rot else 0
         x = ops.resolved(x)
         n = x.shape[0]
-        down = ops.linear(x, self.w_down)  # query latent | latent | shared rotated key part | gates
+        down = ops.linear(x, self.w_down)  # query latent (or queries) | latent | shared rotated key part | gates
+        q_cols = self.q_rank or H * (d + r)
         # the latent is normed, the shared part rotated, and the row goes to its page as one key
         ops.head_prepare(
-            down[:, self.q_rank :], 0, 1, R + r, 0, k_norm=self.kv_norm, norm_dims=R, eps=self.norm_eps, cos_sin=table,
+            down[:, q_cols:], 0, 1, R + r, 0, k_norm=self.kv_norm, norm_dims=R, eps=self.norm_eps, cos_sin=table,
             rot_offset=R, rot_dims=r, pairing=pairing, k_pages=cache.k_pages if cache.writes else None,
             slot_mapping=ctx.slot_mappings[g] if cache.writes else None, page_size=cache.page_size if cache.writes else 0,
         )
-        cq = ops.rmsnorm_columns(down[:, : self.q_rank], self.q_norm, self.norm_eps, x.dtype)
-        q = ops.linear(cq, self.w_uq)  # [n, H * (d + r)]
+        if self.q_rank:
+            cq = ops.rmsnorm_columns(down[:, : self.q_rank], self.q_norm, self.norm_eps, x.dtype)
+            q = ops.linear(cq, self.w_uq)  # [n, H * (d + r)]
+        else:
+            q = down[:, :q_cols]
         if r > 0:
             ops.head_prepare(q, H, 0, d + r, 0, cos_sin=table, rot_offset=d, rot_dims=r, pairing=pairing)
         q_lat = self._per_head(q.view(n, H, d + r)[:, :, :d], self.w_uk_t)       # [H, n, R]
         queries = ops.pack_heads(q_lat, q, d + r, d, r)                           # [n, H * (R + r)]
         mixed = self._mixed_latents(queries, n, ctx, cache)                       # [n, H, R]
         heads = self._per_head(mixed, self.w_uv)                                  # [H, n, dv]
-        gates = down[:, self.q_rank + R + r :] if self.head_gate else None
+        gates = down[:, q_cols + R + r :] if self.head_gate else None
         out = ops.unpack_heads_gate(heads.contiguous(), gates)
         return ops.linear_to_sum(out, self.wo, may_wait=True)

@@ -56,8 +56,8 @@ class Model:
         for layer, nexts in followers.items():
             only = next(iter(nexts)) if len(nexts) == 1 else None
             self.blocks[layer].expects(self.blocks[only] if only is not None else None)
-        # per run: (slot of a mixer, key of its cache entry, whether the run owns the entry)
-        self._run_caches: List[List[Tuple[str, Tuple[int, str], bool]]] = []
+        # per run: (slot of a mixer, name of one of the things it keeps or None, key of the cache entry, whether the run owns the entry)
+        self._run_caches: List[List[tuple]] = []
         for run_id, run in enumerate(spec.order):
             src = run_id if run.cache_from is None else run.cache_from
             if run.cache_from is not None:
@@ -68,7 +68,23 @@ class Model:
                         f"order[{run_id}] borrows the cache of order[{src}], whose layer has no mixer in the "
                         f"slots {sorted(mine - theirs)}"
                     )
-            self._run_caches.append([(slot, (src, slot), run.cache_from is None) for slot in self.blocks[run.layer].mixers()])
+            entries = []
+            for slot, mixer in self.blocks[run.layer].mixers().items():
+                need = mixer.cache_need()
+                if not isinstance(need, dict):
+                    entries.append((slot, None, (src, slot), run.cache_from is None))
+                    continue
+                # a mixer that keeps several things: in a run that borrows, the pages are the other run's and what
+                # else the mixer keeps (state) is its own; what only the other run's mixer has is borrowed too
+                names = dict(need)
+                theirs = {}
+                if run.cache_from is not None:
+                    other = self.blocks[spec.order[src].layer].mixers()[slot].cache_need()
+                    theirs = dict(other) if isinstance(other, dict) else {}
+                for name in list(names) + [n for n in theirs if n not in names]:
+                    borrowed = run.cache_from is not None and name in theirs and (name not in names or hasattr(names[name], "num_kv_heads"))
+                    entries.append((slot, name, (src if borrowed else run_id, slot, name), not borrowed))
+            self._run_caches.append(entries)
 
     def all_parts(self) -> List[Part]:
         """Every part of the model, blocks and their sub-parts included."""
@@ -141,10 +157,12 @@ class Model:
         """``((run id, slot), need)`` for every mixer of every run that owns a cache entry."""
         needs = []
         for run_id, run in enumerate(self.spec.order):
-            if run.cache_from is not None:
-                continue
-            for slot, mixer in self.blocks[run.layer].mixers().items():
-                needs.append(((run_id, slot), mixer.cache_need()))
+            mixers = self.blocks[run.layer].mixers()
+            for slot, name, key, owns in self._run_caches[run_id]:
+                if not owns or key[0] != run_id:
+                    continue
+                need = mixers[slot].cache_need()
+                needs.append((key, need if name is None else need[name]))
         return needs
 
     # ------------------------------------------------------------------ one step
@@ -153,7 +171,12 @@ class Model:
         h = self.embedding.forward(ctx.tokens)
         delta = None
         for run, entries in zip(self.spec.order, self._run_caches):
-            views = {slot: cache.view(key, writes) for slot, key, writes in entries}
+            views = {}
+            for slot, name, key, writes in entries:
+                if name is None:
+                    views[slot] = cache.view(key, writes)
+                else:
+                    views.setdefault(slot, {})[name] = cache.view(key, writes)
             h, delta = self.blocks[run.layer].forward(h, delta, ctx, views)
         if ctx.logit_rows.numel() == 0:
             return torch.empty((0, self.spec.vocab_size), dtype=torch.float32, device=h.device)

@@ -160,3 +160,60 @@ class LayerNorm(Norm):
 
     def forward_rows(self, h: torch.Tensor, delta, rows: torch.Tensor) -> torch.Tensor:
         return ops.layernorm(h, self.weight, self.bias, self.eps, self.out_dtype, delta=self.delta(delta), rows=rows)
+
+
+@NORMS.register("dynamic_tanh")
+class DynamicTanh(Norm):
+    """``y = tanh(alpha x) * weight + bias`` with one learned number ``alpha``: a norm that takes no mean and no
+    variance.  It reads a 32-bit residual stream, or several (``[S, n, D]``: hyper-connections), of which it takes a
+    weighted sum first, and hands on rows of the model's dtype; everything is worked out in 32-bit.  A block over
+    several streams calls ``read`` (the weighted sum and the norm, optionally behind a branch's write into the
+    streams: one kernel); everybody else ``forward`` / ``forward_rows``, which take several streams as their plain sum."""
+
+    graph_safe = True
+
+    def __init__(self, size: int):
+        self.size = size
+        self.weight: Optional[torch.Tensor] = None
+        self.bias: Optional[torch.Tensor] = None
+        self.alpha: Optional[torch.Tensor] = None
+        self.out_dtype: Optional[torch.dtype] = None
+
+    def param_specs(self) -> Dict[str, ParamSpec]:
+        # (kind "matrix": the vectors follow the model's dtype, which is the dtype of the normed rows)
+        return {"weight": ParamSpec((self.size,), kind="matrix", init="ones"), "bias": ParamSpec((self.size,), kind="matrix", init="zeros"),
+                "alpha": ParamSpec((), kind="matrix", init="fraction")}
+
+    def bind(self, tensors: Dict[str, torch.Tensor]) -> None:
+        self.out_dtype = tensors["weight"].dtype
+        self.weight = tensors["weight"].float().contiguous()
+        self.bias = tensors["bias"].float().contiguous()
+        self.alpha = tensors["alpha"].float().reshape(1).contiguous()
+
+    def read(self, streams: torch.Tensor, read_weights: Optional[torch.Tensor], branch=None, mix=None, out_weights=None,
+             rows: Optional[torch.Tensor] = None) -> torch.Tensor:
+        """The normed weighted sum of ``streams`` [S, n, D] (``read_weights`` None: the plain sum; ``rows``: of those
+        tokens only), taken after ``branch`` has gone into the streams through ``mix`` and ``out_weights``, if given."""
+        return ops.streams_update(streams, branch=branch, mix=mix, out_weights=out_weights, read_weights=read_weights,
+                                  alpha=self.alpha, weight=self.weight, bias=self.bias, rows=rows, out_dtype=self.out_dtype)
+
+    @staticmethod
+    def _streams(h: torch.Tensor) -> torch.Tensor:
+        if h.dtype != torch.float32:
+            raise ValueError("dynamic_tanh: the residual stream is 32-bit")
+        return h if h.dim() == 3 else h.unsqueeze(0)
+
+    def forward(self, x: torch.Tensor) -> torch.Tensor:
+        return self.read(self._streams(x), None)
+
+    def forward_add(self, h: torch.Tensor, delta):
+        if delta is not None:
+            if h.dim() == 3:
+                raise ValueError("dynamic_tanh: a sum that is not applied yet cannot be added to several streams")
+            h = h + ops.resolved(delta).float()
+        return h, self.forward(h)
+
+    def forward_rows(self, h: torch.Tensor, delta, rows: torch.Tensor) -> torch.Tensor:
+        if delta is not None:
+            h, _ = self.forward_add(h, delta)
+        return self.read(self._streams(h), None, rows=rows)

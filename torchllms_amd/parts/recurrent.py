@@ -257,3 +257,61 @@ class MatrixMemory(Mixer):
                               self.gate_cap, self.norm_w, self.norm_eps, cache.tensor, 0, ctx.qo_indptr, ctx.slot_ids,
                               self.H, self.dk, self.dv)
         return ops.linear_to_sum(y, self.w_o)
+
+
+@MIXERS.register("gated_linear")
+class GatedLinearAttention(Mixer):
+    """Gated linear attention.  ``q`` (times head_dim^-1/2) and ``k`` (``num_heads`` heads of ``head_dim``) and ``v``
+    (heads of ``v_head_dim``) are projections of the input.  Every key channel has a decay
+    ``alpha = sigmoid(W_a2 (W_a1 h) + b_a2) ** (1 / tau)`` with ``decay_rank`` numbers between the two matrices.  Per head
+    the state, zero at the start, goes ``S <- diag(alpha) S + k v^T`` (the decay acts on the rows that belong to key
+    channels) and ``o = S^T q``; o is divided by its root mean square over v_head_dim, multiplied by the weight ``norm``
+    (shared by the heads) and by ``silu(W_g h)``, then projected by W_o.  Decays, the state and the norm are 32-bit.
+    The recurrence runs in the delta rule's kernels under their plain rule."""
+
+    graph_safe = True
+
+    def __init__(self, hidden_size: int, num_heads: int, head_dim: int, v_head_dim: int, tau: float, decay_rank: int, norm_eps: float):
+        for name, v in (("num_heads", num_heads), ("head_dim", head_dim), ("v_head_dim", v_head_dim), ("decay_rank", decay_rank)):
+            if not isinstance(v, int) or v <= 0:
+                raise ValueError(f"gated_linear: {name} must be a positive integer, got {v!r}")
+        if not float(tau) > 0:
+            raise ValueError(f"gated_linear: tau must be positive, got {tau!r}")
+        self.hidden_size, self.H, self.dk, self.dv, self.rank = hidden_size, num_heads, head_dim, v_head_dim, decay_rank
+        self.tau, self.norm_eps = float(tau), float(norm_eps)
+        self.w_all = self.w_a2 = self.w_o = self.a_bias = self.norm_w = None
+
+    def param_specs(self) -> Dict[str, ParamSpec]:
+        d, qk, v = self.hidden_size, self.H * self.dk, self.H * self.dv
+        return {
+            "q": ParamSpec((qk, d)), "k": ParamSpec((qk, d)), "v": ParamSpec((v, d)), "g": ParamSpec((v, d)),
+            "a1": ParamSpec((self.rank, d)), "a2": ParamSpec((qk, self.rank), init="wide"), "a2.b": ParamSpec((qk,), init="zeros"),
+            "norm": ParamSpec((self.dv,), init="ones"), "o": ParamSpec((d, v)),
+        }
+
+    def check_sizes(self, dtype: torch.dtype) -> None:
+        if self.dk > 256:
+            raise ValueError(f"gated_linear: keys of {self.dk} channels; the kernel takes up to 256 (values: any number)")
+
+    def cache_need(self):
+        return StateNeed(shape=(self.H * self.dv * self.dk,), dtype="float32")
+
+    def bind(self, tensors: Dict[str, torch.Tensor]) -> None:
+        # one projection [q | k | v | output gate | the decay's first matrix]: a single product per step
+        self.w_all = torch.cat([tensors[n] for n in ("q", "k", "v", "g", "a1")], dim=0).contiguous()
+        self.w_a2 = tensors["a2"].contiguous()
+        self.a_bias = tensors["a2.b"].float().contiguous()
+        self.norm_w = tensors["norm"].float().contiguous()
+        self.w_o = tensors["o"].contiguous()
+
+    def linear_weights(self):
+        return [self.w_all, (self.w_a2, "plain", torch.float32), (self.w_o, "sum")]
+
+    def forward(self, x, ctx, cache):
+        qk, v = self.H * self.dk, self.H * self.dv
+        c = 2 * qk + v
+        proj = ops.linear(ops.resolved(x), self.w_all)
+        pre = ops.linear(proj[:, c + v : c + v + self.rank], self.w_a2, out_dtype=torch.float32)
+        y = ops.gated_linear(proj[:, :c], pre, self.a_bias, 1.0 / self.tau, proj, c, self.norm_w, self.norm_eps, cache.tensor, 0,
+                             ctx.qo_indptr, ctx.slot_ids, self.H, self.dk, self.dv)
+        return ops.linear_to_sum(y, self.w_o)

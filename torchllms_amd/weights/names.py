@@ -224,3 +224,44 @@ def kepevik_name_rules(cfg) -> List[NameRule]:
             rules += [NameRule(p + "left." + ext, f"l{i}.left." + own) for ext, own in left.items()]
             rules += [NameRule(p + "right." + n, f"l{i}.right." + n) for n in right]
     return rules
+
+
+def nosuzen_name_rules(cfg) -> List[NameRule]:
+    """Nosuzen checkpoints name a layer's tensors ``l<i>.norm1`` and ``l<i>.norm2`` (with ``.b`` and ``.alpha`` beside the
+    weight), ``l<i>.hc1.{in,out,mix}`` and ``hc2`` (the streams' read, write and mixing weights of the two sublayers),
+    ``l<i>.mix.<tensor>`` (a parallel layer: ``mix.left.<tensor>`` and ``mix.right.<tensor>``; a convolution's taps are
+    ``<tensor>.conv``, a norm inside a mixer ``<tensor>.norm``, a bias ``<tensor>.b``) and ``l<i>.mlp.e<j>.{gate,up,down}``,
+    ``mlp.router``, ``mlp.shared.{gate,up,down}``; beside them ``embed``, ``final.norm`` (+ ``.b``, ``.alpha``) and ``head``."""
+    L = "l{}."
+    rules = [
+        NameRule("embed", "embed.weight"),
+        NameRule("head", "head.weight"),
+        NameRule("final.norm", "final_norm.weight"),
+        NameRule("final.norm.b", "final_norm.bias"),
+        NameRule("final.norm.alpha", "final_norm.alpha"),
+        NameRule(L + "mlp.router", L + "mlp.router.weight"),
+        NameRule(L + "mlp.e{}.gate", L + "mlp.experts.{}.w1.weight"),
+        NameRule(L + "mlp.e{}.up", L + "mlp.experts.{}.w3.weight"),
+        NameRule(L + "mlp.e{}.down", L + "mlp.experts.{}.w2.weight"),
+        NameRule(L + "mlp.shared.gate", L + "mlp.shared.w1.weight"),
+        NameRule(L + "mlp.shared.up", L + "mlp.shared.w3.weight"),
+        NameRule(L + "mlp.shared.down", L + "mlp.shared.w2.weight"),
+    ]
+    for q in ("1", "2"):
+        rules += [NameRule(L + "norm" + q, L + "norm" + q + ".weight"), NameRule(L + "norm" + q + ".b", L + "norm" + q + ".bias"),
+                  NameRule(L + "norm" + q + ".alpha", L + "norm" + q + ".alpha")]
+        rules += [NameRule(L + "hc" + q + "." + n, L + "hc" + q + "." + n) for n in ("in", "out", "mix")]
+    differential = ["q", "k", "v", "q.conv", "k.conv", "v.conv", "lq1", "lk1", "lq2", "lk2", "o"]
+    latent = {"q": "q.weight", "dkv": "dkv.weight", "dkv.norm": "dkv_norm.weight", "uk": "uk.weight", "uv": "uv.weight", "o": "wo.weight"}
+    left = {"q": "wq.weight", "k": "wk.weight", "v": "wv.weight", "q.norm": "q_norm.weight", "k.norm": "k_norm.weight", "o": "wo.weight"}
+    right = ["q", "k", "v", "g", "o", "norm", "a1", "a2", "a2.b"]
+    for i, layer in enumerate(cfg.layers):
+        p = f"l{i}.mix."
+        if layer.type == "attention":
+            rules += [NameRule(p + n, p + n) for n in differential]
+        elif layer.type == "latent_attention":
+            rules += [NameRule(p + ext, p + own) for ext, own in latent.items()]
+        else:
+            rules += [NameRule(p + "left." + ext, f"l{i}.left." + own) for ext, own in left.items()]
+            rules += [NameRule(p + "right." + n, f"l{i}.right." + n) for n in right]
+    return rules

@@ -50,6 +50,9 @@ def random_tensor(name: str, spec: ParamSpec, seed: int, dtype: torch.dtype, nor
     elif spec.init == "fraction":
         # a mixing factor between two things: well inside (0, 1), so that both show
         t = torch.empty(spec.shape, dtype=torch.float32, device=device).uniform_(0.25, 0.75, generator=gen)
+    elif spec.init == "near_identity":
+        # a square matrix that mixes a few things among themselves: the identity and a little of everything
+        t = torch.eye(spec.shape[0], dtype=torch.float32, device=device) + torch.empty(spec.shape, dtype=torch.float32, device=device).uniform_(-0.15, 0.15, generator=gen)
     elif spec.init == "zeros":
         t = torch.zeros(spec.shape, dtype=torch.float32, device=device)
         if norm_jitter > 0:
