@@ -61,6 +61,8 @@ def _sizes(where: str, d, keys) -> Dict[str, Any]:
     for k in keys:
         if k in _NUMBERS:
             _number(where, k, d[k])
+        elif k == "rot_dim":
+            _count(where, k, d[k])  # (a latent layer may rotate nothing)
         elif k not in ("rot", "mask"):
             _positive_int(where, k, d[k])
     return dict(d)
