@@ -2,7 +2,7 @@
 bfloat16 weights, synthetic token ids.
 
     python bench.py [--gpus 1] [--steps K] [--warmup W] [--batch 8] [--context 8192] [--layers L]
-                    [--shape 8b|1b|70b] [--workload decode|serve|peaks|small-kernels|attention|products|taluvik|vobolorn|kepevik]
+                    [--shape 8b|1b|70b] [--workload decode|serve|peaks|small-kernels|attention|products|taluvik|vobolorn|kepevik|nosuzen]
 
 Everything runs through the generation loop: the scheduler admits the requests, cuts their prompts
 into portions under its token budget, and plans every decode step; the step function runs it; the
@@ -28,6 +28,9 @@ a read of 4 GiB with 16-byte loads, a device copy, a loop of MFMA instructions o
 library's large matrix product.  ``--workload small-kernels`` times what a norm kernel adds to a
 replayed graph of large products, without a profiler (under rocprofv3 no dispatch is shorter than
 about 4.6 us, an empty kernel included, so a kernel trace overstates the small kernels of a step).
+``--workload nosuzen``: prefill and decode of a Nosuzen model (several residual streams, differential attention behind short
+convolutions with kept first keys, attention through a latent, attention beside gated linear attention, routed
+feed-forwards with grouped routers) beside a Kepevik model of the same layer sizes.
 ``--workload kepevik``: prefill and decode of a Kepevik model (matrix memory, attention beside a delta rule with a
 decay per key channel, routed feed-forwards) beside a Taluvik model of the same layer sizes.
 ``--workload taluvik``: prefill and decode of a Taluvik model (chunked attention with sinks, gated delta
@@ -86,8 +89,8 @@ def parse_args(argv=None):
     p.add_argument("--points", default="1,64", help="further decode batch sizes, comma separated ('' for none)")
     p.add_argument("--page-size", type=int, default=16)
     p.add_argument("--shape", default="8b", choices=sorted(SHAPES), help="layer sizes (default: the headline's)")
-    p.add_argument("--workload", default="decode", choices=["decode", "serve", "peaks", "small-kernels", "attention", "products", "taluvik", "vobolorn", "kepevik"])
-    p.add_argument("--only", default=None, choices=["taluvik", "vobolorn", "kepevik", "llama"], help="taluvik, vobolorn, kepevik: measure one of the two models only")
+    p.add_argument("--workload", default="decode", choices=["decode", "serve", "peaks", "small-kernels", "attention", "products", "taluvik", "vobolorn", "kepevik", "nosuzen"])
+    p.add_argument("--only", default=None, choices=["taluvik", "vobolorn", "kepevik", "nosuzen", "llama"], help="taluvik, vobolorn, kepevik, nosuzen: measure one of the two models only")
     p.add_argument("--token-budget", type=int, default=8192, help="tokens a step may hold (the scheduler cuts prompts to it)")
     p.add_argument("--no-reference-workload", action="store_true",
                    help="leave out the reference's benchmark (2,048-token prompts, 256 new tokens at batch 1, 8, 64)")
@@ -358,6 +361,41 @@ def kepevik_config(shape: dict, n_layers: int) -> dict:
                         "mlp": {"kind": "dense", "ff": ff} if i == 0 else moe} for i in range(n_layers)]}
 
 
+def nosuzen_config(shape: dict, n_layers: int) -> dict:
+    """A Nosuzen configuration with the layer sizes of ``shape`` (a Llama configuration): the same width and head size,
+    four residual streams.  Four kinds of layer take turns: differential attention with half the shape's heads (two
+    maps each, values twice as wide, so its projections have the shape's sizes) behind convolutions over four taps,
+    a window of 4,096 that keeps the first 64 positions; attention (the shape's heads, YaRN) beside gated linear
+    attention with half as many heads and 64 numbers inside its decay; differential attention that reads the keys and
+    values of the one two layers before; attention through a latent of 192 channels beside 64 rotated ones.  Every
+    feed-forward is a mixture of eight experts of a quarter of the shape's inner width in four groups of which two
+    stay, a token uses two, beside a shared expert of a quarter of that width."""
+    D, H, G, dh, ff = shape["hidden_size"], shape["num_attention_heads"], shape["num_key_value_heads"], shape["head_dim"], shape["intermediate_size"]
+    yarn = {"factor": 8.0, "original": 8192, "fast": 32.0, "slow": 1.0}
+    differential = {"heads": max(H // 2, 1), "kv_heads": max(G // 2, 1), "dim": dh, "vdim": 2 * dh, "scale": dh ** -0.5, "diff": 0.6, "conv": 4,
+                    "rot": {"dims": dh, "base": shape["rope_theta"]}, "mask": {"size": 4096, "keep_first": 64}}
+    pair = {"left": {"heads": H, "kv_heads": G, "dim": dh, "vdim": dh, "scale": dh ** -0.5, "rot": {"dims": dh // 2, "base": shape["rope_theta"], "scaling": yarn},
+                     "mask": {"size": 4096, "keep_first": 64}},
+            "right": {"heads": max(H // 2, 1), "dim": dh, "vdim": dh, "tau": 16.0, "decay_rank": 64},
+            "left_scale": 0.6, "right_scale": 0.5}
+    through_latent = {"heads": H, "dim": dh, "rot_dim": 64, "vdim": dh, "kv_rank": 192, "scale": (dh + 64) ** -0.5,
+                      "rot": {"dims": 64, "base": 10000.0, "scaling": yarn}, "mask": {"size": 4096}}
+    moe = {"kind": "moe", "expert": {"ff": ff // 4}, "router": {"experts": 8, "top": 2, "scale": 2.0, "groups": {"count": 4, "keep": 2}}, "shared": {"ff": ff // 4}}
+    layers = []
+    for i in range(n_layers):
+        kind = i % 4
+        if kind == 0:
+            layers.append({"type": "attention", "mixer": differential, "mlp": moe})
+        elif kind == 1:
+            layers.append({"type": "parallel", "mixer": pair, "mlp": moe})
+        elif kind == 2:
+            layers.append({"type": "attention", "mixer": dict(differential, kv_from=i - 2), "mlp": moe})
+        else:
+            layers.append({"type": "latent_attention", "mixer": through_latent, "mlp": moe})
+    return {"architecture": "Nosuzen", "vocab": shape["vocab_size"], "width": D, "streams": 4, "embedding": {"scale": 1.0}, "norm": {"eps": 1e-6},
+            "layers": layers}
+
+
 def taluvik_run(args, shape) -> int:
     """Prefill and decode of a Taluvik (or, ``--workload vobolorn``, a Vobolorn) model beside a Llama model of the
     same layer sizes and number of layers, both with random weights, both through the same engine, scheduler and
@@ -373,9 +411,17 @@ def taluvik_run(args, shape) -> int:
     n_layers = args.layers or 8
     batches = [args.batch] + [int(b) for b in args.points.split(",") if b]
     pages_per_req = -(-max(args.context, args.prefill_tokens) // args.page_size) + 1
-    design = {"vobolorn": "Vobolorn", "kepevik": "Kepevik"}.get(args.workload, "Taluvik")
+    design = {"vobolorn": "Vobolorn", "kepevik": "Kepevik", "nosuzen": "Nosuzen"}.get(args.workload, "Taluvik")
     beside = "Llama"
-    if args.workload == "kepevik":
+    if args.workload == "nosuzen":
+        # beside the design nearest to it: Kepevik, whose layers hold attention beside a recurrence and routed feed-forwards too
+        from torchllms_amd.config.kepevik import KepevikConfig
+        from torchllms_amd.config.nosuzen import NosuzenConfig
+
+        beside = "Kepevik"
+        configs = {"nosuzen": NosuzenConfig.from_dict(nosuzen_config(shape, n_layers)),
+                   "kepevik": KepevikConfig.from_dict(kepevik_config(shape, n_layers))}
+    elif args.workload == "kepevik":
         # beside the design nearest to it: Taluvik, whose layers hold a delta rule, attention and a recurrence too
         from torchllms_amd.config.kepevik import KepevikConfig
 
@@ -650,7 +696,7 @@ def main(argv=None) -> int:
         return products_run(args, shape)
     if args.workload == "peaks":
         return peaks_run(args)
-    if args.workload in ("taluvik", "vobolorn", "kepevik"):
+    if args.workload in ("taluvik", "vobolorn", "kepevik", "nosuzen"):
         return taluvik_run(args, shape)
     import torch
 

@@ -275,6 +275,70 @@ def test_plain_attention_with_kept_first_keys_and_fewer_value_heads(Hq, Hk, Hv, 
             assert (one.float().view(Hq, dv).double() - ref).abs().max() < tol * max(1.0, float(ref.abs().max()))
 
 
+@pytest.mark.parametrize("Hq,Hk,Hv,d,dv,page,window,keep", [
+    (8, 2, 2, 128, 128, 16, 200, 20), (4, 4, 2, 64, 128, 16, 70, 64), (8, 4, 2, 128, 256, 32, 136, 70), (2, 2, 1, 32, 96, 16, 33, 5),
+    (16, 1, 1, 64, 64, 8, 1000, 3), (4, 2, 1, 256, 256, 16, 100, 100), (6, 2, 2, 128, 128, 16, 64, 0)])
+def test_matrix_core_attention_with_kept_first_keys_and_wide_values(Hq, Hk, Hv, d, dv, page, window, keep):
+    """The split-KV decode kernel and the tiled prefill kernel against the plain kernel (which the test above holds
+    against the formulas): a window that keeps first positions, values with fewer heads than the keys and rows that
+    are a multiple of the keys' head size (worked off in calls of one head size each); queries that like the keys at
+    the window's edges and at the end of the kept positions; single tokens at many positions, and portions of a
+    prompt that begin before, at and behind the window's first full reach, behind a prefix in the cache."""
+    from torchllms_amd.kernels import ops
+
+    gen = torch.Generator().manual_seed(Hq + d + window)
+    n, scale = 700, 0.7 / d ** 0.5
+    keys = torch.randn((n, Hk, d), generator=gen).to(torch.bfloat16)
+    values = torch.randn((n, Hv, dv), generator=gen).to(torch.bfloat16)
+    k_pages, v_pages, table = _paged(keys.float(), values.float(), page, 2 * (n // page) + 9, gen)
+    kp, vp = k_pages.to(DEV, torch.bfloat16), v_pages.to(DEV, torch.bfloat16)
+    bt = table.to(DEV).view(1, -1)
+
+    def queries_for(positions):
+        q = torch.randn((len(positions), Hq, d), generator=gen)
+        for i, p in enumerate(positions):
+            edge = [j for j in (p - window + 1, p - window, keep - 1, keep) if 0 <= j <= p]
+            for h in range(Hq):
+                q[i, h] = sum(keys[j, h // (Hq // Hk)].float() for j in edge) * (5.0 / (scale * d)) + q[i, h]
+        return q.reshape(len(positions), Hq * d).to(DEV, torch.bfloat16)
+
+    kw = dict(keep_first=keep, value_heads=Hv)
+    # single tokens
+    positions = [0, 1, 15, 16, keep, keep + 1, window - 1, window, window + 1, window + keep - 1, window + keep, window + keep + 17, 300, 511, 512, 699]
+    positions = sorted({min(max(p, 0), n - 1) for p in positions})
+    q = queries_for(positions)
+    pos = torch.tensor(positions, dtype=torch.int32, device=DEV)
+    seq = torch.zeros(len(positions), dtype=torch.int32, device=DEV)
+    want = ops.attention_generic(q, Hq, Hk, d, kp, vp, seq, pos, bt, window, scale, v_head_dim=dv, **kw).float()
+    for split in (None, 64, 128):
+        got = torch.zeros((len(positions), Hq * dv), dtype=torch.bfloat16, device=DEV)
+        for at in range(0, dv, d):
+            ops.attention_decode(q, Hq, Hk, d, kp, vp, seq, pos, bt, window, scale, min(max(positions) + 1, window + 15), out=got,
+                                 split_size=split, v_offset=at, **kw)
+        assert (got.float() - want).abs().max() < 3e-2 * max(1.0, float(want.abs().max())), (split, (got.float() - want).abs().max())
+    # portions of a prompt behind what the cache holds already
+    if not ops.prefill_attention_supported(torch.bfloat16, Hq, Hk, d, page):
+        return
+    qpt = ops.prefill_queries_per_tile(Hq, Hk, d)
+    for first, count in ((0, 700), (0, 40), (keep + 3, 90), (window - 5, 130), (window + keep - 20, 77), (500, 200), (690, 10)):
+        if first + count > n:  # (only what the cache holds)
+            continue
+        ps = list(range(first, first + count))
+        q = queries_for(ps)
+        qo = torch.tensor([0, count], dtype=torch.int32, device=DEV)
+        kv = torch.tensor([first + count], dtype=torch.int32, device=DEV)
+        rows, q0s = ops.prefill_tiles([0, count], 0, 1, qpt, [first + count], window)
+        tiles = torch.tensor([rows, q0s], dtype=torch.int32, device=DEV)
+        want = ops.attention_generic(q, Hq, Hk, d, kp, vp, torch.zeros(count, dtype=torch.int32, device=DEV),
+                                     torch.tensor(ps, dtype=torch.int32, device=DEV), bt, window, scale, v_head_dim=dv, **kw).float()
+        for groups in (1, 2):
+            got = torch.zeros((count, Hq * dv), dtype=torch.bfloat16, device=DEV)
+            for at in range(0, dv, d):
+                ops.attention_prefill(q, Hq, Hk, d, kp, vp, qo, kv, bt, tiles[0], tiles[1], window, scale, got, key_groups=groups, v_offset=at, **kw)
+            err = (got.float() - want).abs().max(dim=1).values
+            assert float(err.max()) < 3e-2 * max(1.0, float(want.abs().max())), (first, count, groups, int(err.argmax()) + first, float(err.max()))
+
+
 @pytest.mark.parametrize("S,D,n", [(3, 256, 70), (1, 64, 5), (4, 50, 33), (8, 36, 2)])
 def test_streams_kernel_against_the_formulas(S, D, n):
     from torchllms_amd.kernels import ops

@@ -76,6 +76,12 @@ struct DecodeArgs {
   int page_size;
   int page_shift;  // log2(page_size) when that is a power of two, else -1
   int window;
+  int keep_first;     // > 0: behind a window (or chunk) a query also sees the first keep_first positions
+  int n_v_heads;      // heads of the value pages: key head g reads value head g % n_v_heads
+  int v_pitch;        // elements of a value row in the pages (>= DH), of which DH from v_offset are this call's
+  int v_offset;
+  int out_pitch;      // elements between two heads' outputs of a token, of which DH from out_offset are this call's
+  int out_offset;
   int chunk;          // > 0: a query sees only the keys of its own chunk of that many positions
   float scale_log2e;  // softmax scale * log2(e): probabilities are exp2 of scaled differences
   float cap_log2e;    // > 0: scores are capped, cap * tanh(score / cap); this is cap * log2(e) ...
@@ -150,9 +156,15 @@ __global__ void __launch_bounds__(kWaves* kWave, TL_DECODE_MIN_WAVES) attn_decod
   const int p = a.positions[t];
   const int lo = first_key(p, a.window, a.chunk);
   const int lo_al = lo & ~(kTile - 1);
-  const int split_begin = lo_al + split * a.split_size;
-  if (split_begin > p) return;  // whole block: nothing in this split
-  const int split_end = min(split_begin + a.split_size - 1, p);  // last key, inclusive
+  // The keys a query sees are counted through: first the kept first positions 0 .. n_keep - 1 (rounded up to whole
+  // tiles), then the positions from lo_al to p.  Splits, tiles and the prefetch walk this count; `key_of` says which
+  // position a count stands for (counts that stand for nothing a query sees are clamped to one it does see, and masked).
+  const int n_keep = min(a.keep_first, lo);
+  const int keep_al = (n_keep + kTile - 1) & ~(kTile - 1);
+  const int n_counts = keep_al + (p - lo_al + 1);
+  const int split_begin = split * a.split_size;
+  if (split_begin >= n_counts) return;  // whole block: nothing in this split
+  const int split_end = min(split_begin + a.split_size - 1, n_counts - 1);  // last count, inclusive
   const int32_t* bt = a.block_table + (size_t)b * a.bt_stride;
   const int R = a.group;
   const size_t head_elems = (size_t)a.page_size * DH;
@@ -177,11 +189,20 @@ __global__ void __launch_bounds__(kWaves* kWave, TL_DECODE_MIN_WAVES) attn_decod
   // Keys are clamped to the split's own range: the prefetch that runs past the split's end then
   // reads one row that the block has read already, not rows of the next split, which another block
   // reads (a quarter more traffic at splits of 256 keys).
-  auto clamp_key = [&](int key) { return key < lo ? lo : (key > split_end ? split_end : key); };
+  auto clamp_key = [&](int count) {
+    count = count > split_end ? split_end : count;
+    if (count < keep_al) return count < n_keep ? count : n_keep - 1;
+    const int key = lo_al + (count - keep_al);
+    return key < lo ? lo : key;
+  };
   auto block_of = [&](int key) { return kPow2Pages ? key >> a.page_shift : key / a.page_size; };
   auto offset_of = [&](int key) { return kPow2Pages ? key & (a.page_size - 1) : key % a.page_size; };
   auto row_ptr = [&](const bf16_t* pages, int page, int key) {
     return pages + ((size_t)page * a.n_kv_heads + kvh) * head_elems + (size_t)offset_of(key) * DH;
+  };
+  const int vh = kvh % a.n_v_heads;
+  auto value_ptr = [&](int page, int key) {
+    return a.v_pages + (((size_t)page * a.n_v_heads + vh) * a.page_size + (size_t)offset_of(key)) * a.v_pitch + a.v_offset;
   };
 
   // The page ids of a tile's rows: one for the lane's key row, four for its value rows.  They are
@@ -220,7 +241,7 @@ __global__ void __launch_bounds__(kWaves* kWave, TL_DECODE_MIN_WAVES) attn_decod
   auto load_v = [&](int base, const TilePages& tp) {
 #pragma unroll
     for (int j = 0; j < 4; ++j)
-      load_value_words(row_ptr(a.v_pages, tp.v[j], clamp_key(base + 4 * g4 + j)) + kE * n16, vreg[j]);
+      load_value_words(value_ptr(tp.v[j], clamp_key(base + 4 * g4 + j)) + kE * n16, vreg[j]);
   };
 
   int base = split_begin + wave * kTile;
@@ -247,8 +268,9 @@ __global__ void __launch_bounds__(kWaves* kWave, TL_DECODE_MIN_WAVES) attn_decod
     float tmax = -INFINITY;
 #pragma unroll
     for (int i = 0; i < 4; ++i) {
-      const int key = base + 4 * g4 + i;
-      const bool valid = (key >= lo) & (key <= p);  // bit operation: no branch behind the MFMAs
+      const int count = base + 4 * g4 + i;
+      const int key = lo_al + (count - keep_al);
+      const bool valid = count < keep_al ? count < n_keep : (key >= lo) & (key <= p);  // selects: no branch behind the MFMAs
       float sc = c[i] * a.scale_log2e;
       if (a.cap_log2e > 0.f)  // (the same in every lane)
         sc = a.cap_log2e * (1.0f - 2.0f * __builtin_amdgcn_rcpf(__builtin_amdgcn_exp2f(c[i] * a.two_scale_over_cap_log2e) + 1.0f));
@@ -316,7 +338,7 @@ __global__ void __launch_bounds__(kWaves* kWave, TL_DECODE_MIN_WAVES) attn_decod
     const int qh = kvh * R + h;
     if (a.n_splits == 1) {
       if (a.sinks) L += __builtin_amdgcn_exp2f(a.sinks[qh] * 1.4426950408889634f - M);
-      a.out[(size_t)t * a.out_stride + (size_t)qh * DH + d] = from_f32<bf16_t>(O / L);
+      a.out[(size_t)t * a.out_stride + (size_t)qh * a.out_pitch + a.out_offset + d] = from_f32<bf16_t>(O / L);
     } else {
       const size_t slot = ((size_t)t * a.n_kv_heads * R + qh) * a.n_splits + split;
       a.ws_o[slot * DH + d] = O;
@@ -360,7 +382,8 @@ __global__ void __launch_bounds__(kWave) attn_decode_merge_kernel(DecodeArgs a, 
   fetch(0);
   const int lo = first_key(p, a.window, a.chunk);
   const int lo_al = lo & ~(kTile - 1);
-  const int n_valid = min((p - lo_al) / a.split_size + 1, a.n_splits);
+  const int keep_al = (min(a.keep_first, lo) + kTile - 1) & ~(kTile - 1);
+  const int n_valid = min((keep_al + p - lo_al) / a.split_size + 1, a.n_splits);
   float M = lane < n_valid ? m_mine : -INFINITY;
   for (int s = lane + kWave; s < n_valid; s += kWave) M = fmaxf(M, a.ws_ml[(slot0 + s) * 2]);
   M = wave_max(M);
@@ -387,7 +410,7 @@ __global__ void __launch_bounds__(kWave) attn_decode_merge_kernel(DecodeArgs a, 
 #pragma unroll
   for (int c = 0; c < NC; ++c) {
     const int d = lane + c * kWave;
-    if (d < DH) a.out[(size_t)t * a.out_stride + (size_t)qh * DH + d] = from_f32<bf16_t>(o[c] / L);
+    if (d < DH) a.out[(size_t)t * a.out_stride + (size_t)qh * a.out_pitch + a.out_offset + d] = from_f32<bf16_t>(o[c] / L);
   }
 }
 
@@ -399,17 +422,25 @@ TL_EXPORT int tl_attn_decode_head_dim() { return DH; }
 // softcap > 0 caps the scores, chunk > 0 confines a query to its chunk, sinks (one float per query head, or
 // null) join the denominators.  Every token is one query at positions[t] of request row token_seq[t].  split_size: keys per
 // split (a multiple of 64); n_splits >= ceil(longest visible range / split_size), counted from the
-// 16-aligned first visible key.  ws_o / ws_ml: workspaces (unused when n_splits == 1).
+// 16-aligned first visible key, plus the kept first keys rounded up to 16.  keep_first, n_v_heads (0: n_kv_heads),
+// v_pitch / v_offset and out_pitch / out_offset (0: DH): see DecodeArgs.  ws_o / ws_ml: workspaces (unused when n_splits == 1).
 TL_EXPORT int tl_attn_decode(const void* q, int q_stride, void* out, int out_stride, const void* k_pages,
                              const void* v_pages, const int32_t* token_seq, const int32_t* positions,
                              const int32_t* block_table, int bt_stride, int n_tokens, int n_q_heads,
                              int n_kv_heads, int head_dim, int page_size, int window, float scale,
                              int split_size, int n_splits, float* ws_o, float* ws_ml, float softcap, int chunk,
-                             const float* sinks, hipStream_t stream) {
+                             const float* sinks, int keep_first, int n_v_heads, int v_pitch, int v_offset, int out_pitch,
+                             int out_offset, hipStream_t stream) {
   if (head_dim != DH) return variant_fail(TL_ERR_ARG, "attn_decode: built for head_dim %d, called with %d", DH, head_dim);
   if (n_tokens < 0 || n_q_heads <= 0 || n_kv_heads <= 0 || page_size <= 0 || bt_stride <= 0 || window < 0 || chunk < 0 || softcap < 0)
     return variant_fail(TL_ERR_ARG, "attn_decode: bad sizes");
   if (n_q_heads % n_kv_heads) return variant_fail(TL_ERR_ARG, "attn_decode: %d query heads are not a multiple of %d kv heads", n_q_heads, n_kv_heads);
+  if (n_v_heads <= 0) n_v_heads = n_kv_heads;
+  if (v_pitch <= 0) v_pitch = DH;
+  if (out_pitch <= 0) out_pitch = DH;
+  if (keep_first < 0 || n_kv_heads % n_v_heads || v_offset < 0 || v_offset + DH > v_pitch || out_offset < 0 || out_offset + DH > out_pitch
+      || v_pitch % 8 || v_offset % 8)
+    return variant_fail(TL_ERR_ARG, "attn_decode: kept keys, value heads or the places of values and outputs do not fit");
   const int R = n_q_heads / n_kv_heads;
   constexpr int kMaxGroup = DH <= 128 ? 16 : 8;  // bounded by the block's LDS (64 KB of partial outputs)
   if (R > kMaxGroup) return variant_fail(TL_ERR_UNSUPPORTED, "attn_decode: %d query heads per kv head exceed %d at head_dim %d", R, kMaxGroup, DH);
@@ -428,6 +459,8 @@ TL_EXPORT int tl_attn_decode(const void* q, int q_stride, void* out, int out_str
     if ((1 << sh) == page_size) a.page_shift = sh;
   a.scale_log2e = scale * 1.4426950408889634f;
   a.chunk = chunk; a.sinks = sinks;
+  a.keep_first = keep_first; a.n_v_heads = n_v_heads; a.v_pitch = v_pitch; a.v_offset = v_offset;
+  a.out_pitch = out_pitch; a.out_offset = out_offset;
   a.cap_log2e = softcap > 0 ? softcap * 1.4426950408889634f : 0.f;
   a.two_scale_over_cap_log2e = softcap > 0 ? 2.0f * scale / softcap * 1.4426950408889634f : 0.f;
   a.split_size = split_size; a.n_splits = n_splits; a.ws_o = ws_o; a.ws_ml = ws_ml;

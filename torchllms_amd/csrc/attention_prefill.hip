@@ -98,6 +98,12 @@ struct PrefillArgs {
   int page_size;
   int page_shift;  // log2(page_size)
   int window;
+  int keep_first;  // > 0: behind a window (or chunk) a query also sees the first keep_first positions
+  int n_v_heads;   // heads of the value pages: key head g reads value head g % n_v_heads
+  int v_pitch;     // elements of a value row in the pages (>= DH), of which DH from v_offset are this call's
+  int v_offset;
+  int out_pitch;   // elements between two heads' outputs of a token, of which DH from out_offset are this call's
+  int out_offset;
   int chunk;  // > 0: a query sees only the keys of its own chunk of that many positions
   float scale_log2e;
   float cap_over_scale;             // capped scores: s <- cap * tanh(s * scale / cap), taken on the raw product as
@@ -158,10 +164,11 @@ __device__ __forceinline__ u32x2_t lds_transposed(const bf16_t* src) {
 // of kWaves waves that take the same columns and every second tile of keys each, and add up what
 // they have at the end through LDS: a block's chain of tiles is half as long, which is what a launch
 // needs whose blocks all fit the GPU at once and whose time is therefore that of its longest block.
-// MODE 0: no lower bound and no cap; 1: a lower bound (a window, chunks, or both); 2: a lower bound and capped scores.
+// MODE 0: no lower bound and no cap; 1: a lower bound (a window, chunks, or both); 2: a lower bound and capped scores;
+// 3: a lower bound, and before it the first keep_first positions, which come as tiles of their own ahead of the others.
 template <int RP, int MODE, int GROUPS>
 __global__ void __launch_bounds__(GROUPS * kWaves * kWave, GROUPS == 1 ? 2 : 1) attn_prefill_kernel(PrefillArgs a) {
-  constexpr bool WINDOWED = MODE >= 1, CAPPED = MODE == 2;
+  constexpr bool WINDOWED = MODE >= 1, CAPPED = MODE == 2, KEPT = MODE == 3;
   constexpr int QB = kCols / RP;  // queries per block
 
   const int tile = blockIdx.y;  // the host lists the tiles in the order that balances the launch
@@ -192,6 +199,10 @@ __global__ void __launch_bounds__(GROUPS * kWaves * kWave, GROUPS == 1 ? 2 : 1) 
   const int key_lo = window_lo(pos0 + q0);          // first key any column sees
   const int key_hi = pos0 + q_last;                 // last key any column sees
   const int tile_begin = key_lo & ~(KT - 1);
+  // the kept first positions that some column sees are 0 .. keep_blk - 1 (the last query's are the most): n_keep_tiles
+  // tiles of their own, walked before the tiles from tile_begin on; a column sees a kept key below its own lower bound
+  const int keep_blk = KEPT ? min(a.keep_first, window_lo(pos0 + q_last)) : 0;
+  const int n_keep_tiles = KEPT ? (keep_blk + KT - 1) / KT : 0;
 
   // this lane's columns: col -> (query, head)
   int col_pos[NC], col_lo[NC], col_tok[NC], col_head[NC];
@@ -237,7 +248,10 @@ __global__ void __launch_bounds__(GROUPS * kWaves * kWave, GROUPS == 1 ? 2 : 1) 
   const int blk_lo = key_lo >> a.page_shift, blk_hi = key_hi >> a.page_shift;
   const unsigned page_bytes = (unsigned)a.n_kv_heads * (unsigned)a.page_size * DH * 2;  // all kv heads of a page
   const char* const k_head = reinterpret_cast<const char*>(a.k_pages) + (size_t)kvh * head_elems * 2;  // this kv head's rows in page 0
-  const char* const v_head = reinterpret_cast<const char*>(a.v_pages) + (size_t)kvh * head_elems * 2;
+  const unsigned v_row_bytes = (unsigned)a.v_pitch * 2;
+  const unsigned v_page_bytes = (unsigned)a.n_v_heads * (unsigned)a.page_size * v_row_bytes;
+  const char* const v_head = reinterpret_cast<const char*>(a.v_pages) + ((size_t)(kvh % a.n_v_heads) * a.page_size * a.v_pitch + a.v_offset) * 2;
+  const int keep_blk_hi = keep_blk > 0 ? (keep_blk - 1) >> a.page_shift : 0;
   // The rows of one wave load (64 lanes x 16 bytes: kRowsPerLoad rows) lie in one page (the host sees to
   // it that a page holds at least as many rows, and tiles start at multiples of the tile's size), so a
   // load's page is one number for the wave: it is looked up by a scalar load and the page's address is
@@ -248,11 +262,12 @@ __global__ void __launch_bounds__(GROUPS * kWaves * kWave, GROUPS == 1 ? 2 : 1) 
   struct Rows {
     int page[kLoadsPerWave];
   };
-  auto lookup = [&](int base, Rows& rows) {
+  auto lookup = [&](int base, bool kept, Rows& rows) {
 #pragma unroll
     for (int j = 0; j < kLoadsPerWave; ++j) {
       int blk = (base + (j * kWaves + wave) * kRowsPerLoad) >> a.page_shift;
-      blk = blk < blk_lo ? blk_lo : (blk > blk_hi ? blk_hi : blk);
+      if (KEPT && kept) blk = blk > keep_blk_hi ? keep_blk_hi : blk;  // (the pages of the kept positions are held)
+      else blk = blk < blk_lo ? blk_lo : (blk > blk_hi ? blk_hi : blk);
       rows.page[j] = table[blk];
     }
   };
@@ -262,9 +277,10 @@ __global__ void __launch_bounds__(GROUPS * kWaves * kWave, GROUPS == 1 ? 2 : 1) 
       const int first = (j * kWaves + wave) * kRowsPerLoad;
       const int r = first + lane / kPieces;
       const int piece = (lane % kPieces) ^ (values ? swizzle_v(r) : swizzle(r));
-      const unsigned of_lane = (unsigned)(lane / kPieces) * (DH * 2) + 16 * piece;  // the same for every tile
-      const unsigned in_page = (unsigned)((base + first) & (a.page_size - 1)) * (DH * 2);
-      const char* src = (values ? v_head : k_head) + ((size_t)(unsigned)rows.page[j] * page_bytes + in_page);
+      const unsigned row_bytes = values ? v_row_bytes : (unsigned)(DH * 2);
+      const unsigned of_lane = (unsigned)(lane / kPieces) * row_bytes + 16 * piece;  // the same for every tile
+      const unsigned in_page = (unsigned)((base + first) & (a.page_size - 1)) * row_bytes;
+      const char* src = (values ? v_head : k_head) + ((size_t)(unsigned)rows.page[j] * (values ? v_page_bytes : page_bytes) + in_page);
       __builtin_amdgcn_global_load_lds(reinterpret_cast<const bf16_t*>(src + of_lane),
                                        &tiles[(2 * buffer + (values ? 1 : 0)) * kTileElems + first * DH], 16, 0, 0);
     }
@@ -336,7 +352,7 @@ __global__ void __launch_bounds__(GROUPS * kWaves * kWave, GROUPS == 1 ? 2 : 1) 
   // not see some key of the tile; where every column sees every key the tests are compiled out.
   constexpr float kSlack = 8.f;
   // scores of keys that a column does not see become -inf (plain selects, no short-circuit)
-  auto mask = [&](int base) {
+  auto mask = [&](int base, bool kept) {
 #pragma unroll
     for (int i = 0; i < NC; ++i)
 #pragma unroll
@@ -344,7 +360,8 @@ __global__ void __launch_bounds__(GROUPS * kWaves * kWave, GROUPS == 1 ? 2 : 1) 
 #pragma unroll
         for (int r = 0; r < 4; ++r) {
           const int key = base + 16 * sub + 4 * g4 + r;
-          const bool valid = WINDOWED ? (key >= col_lo[i]) & (key <= col_pos[i]) : key <= col_pos[i];
+          bool valid = WINDOWED ? (key >= col_lo[i]) & (key <= col_pos[i]) : key <= col_pos[i];
+          if (KEPT) valid = kept ? key < min(a.keep_first, col_lo[i]) : valid;
           c[i][sub][r] = valid ? c[i][sub][r] : -INFINITY;
         }
   };
@@ -401,17 +418,21 @@ __global__ void __launch_bounds__(GROUPS * kWaves * kWave, GROUPS == 1 ? 2 : 1) 
 
   // Every wave of the block passes the same number of barriers: with two groups both make as many
   // steps, and the second one's last tile may lie past the last key (its keys are clamped and masked).
-  const int n_steps = ((key_hi - tile_begin) / KT + GROUPS) / GROUPS;
-  auto base_of = [&](int step) { return tile_begin + (step * GROUPS + grp) * KT; };
+  const int n_steps = ((key_hi - tile_begin) / KT + n_keep_tiles + GROUPS) / GROUPS;
+  auto kept_of = [&](int step) { return KEPT && step * GROUPS + grp < n_keep_tiles; };
+  auto base_of = [&](int step) {
+    const int nth = step * GROUPS + grp;
+    return KEPT && nth < n_keep_tiles ? nth * KT : tile_begin + (nth - n_keep_tiles) * KT;
+  };
   auto k_tile = [&](int step) { return tiles + (2 * (step & 1)) * kTileElems; };
   auto v_tile = [&](int step) { return tiles + (2 * (step & 1) + 1) * kTileElems; };
 
   Rows rows_k, rows_v;  // the rows of the next pass's loads: keys of tile step + 2, values of tile step
-  lookup(base_of(0), rows_v);
-  lookup(base_of(1), rows_k);
+  lookup(base_of(0), kept_of(0), rows_v);
+  lookup(base_of(1), kept_of(1), rows_k);
   dma(base_of(0), rows_v, 0, false);  // (tile 0's keys lie where its values do)
   dma(base_of(1), rows_k, 1, false);
-  lookup(base_of(2), rows_k);
+  lookup(base_of(2), kept_of(2), rows_k);
   // the first pass has no tile before it: its output product runs all the same (no branch in a pass),
   // on probabilities of zero and values of zero
 #pragma unroll
@@ -434,8 +455,8 @@ __global__ void __launch_bounds__(GROUPS * kWaves * kWave, GROUPS == 1 ? 2 : 1) 
     __syncthreads();
     dma(base_of(step + 2), rows_k, step & 1, false);  // unconditional (pages are clamped): no wait has to cover a path without it
     dma(base_of(step), rows_v, step & 1, true);
-    lookup(base_of(step + 3), rows_k);  // for the next pass
-    lookup(base_of(step + 1), rows_v);
+    lookup(base_of(step + 3), kept_of(step + 3), rows_k);  // for the next pass
+    lookup(base_of(step + 1), kept_of(step + 1), rows_v);
     bf16x8_t pb[NC][NS / 2];
     float alpha[NC];
     bool moved;
@@ -451,7 +472,7 @@ __global__ void __launch_bounds__(GROUPS * kWaves * kWave, GROUPS == 1 ? 2 : 1) 
           for (int r = 0; r < 4; ++r)
             c[i][sub][r] = a.cap_over_scale * (1.0f - 2.0f * __builtin_amdgcn_rcpf(__builtin_amdgcn_exp2f(c[i][sub][r] * a.two_scale_over_cap_log2e) + 1.0f));
     }
-    if (base + KT - 1 > pos0 + q0 || (WINDOWED && base < window_lo(pos0 + q_last))) mask(base);
+    if (kept_of(step) || base + KT - 1 > pos0 + q0 || (WINDOWED && base < window_lo(pos0 + q_last))) mask(base, kept_of(step));
     softmax(pb, alpha, moved);
     output(v_tile(step - 1), pb_prev);
     if (__any(moved)) rescale(alpha);  // (the same for the whole wave)
@@ -521,7 +542,7 @@ __global__ void __launch_bounds__(GROUPS * kWaves * kWave, GROUPS == 1 ? 2 : 1) 
     if (!col_ok[i]) continue;
     if (a.sinks) l += exp2_fast(a.sinks[col_head[i]] * 1.4426950408889634f - m_run[i]);
     const float inv = 1.0f / l;
-    bf16_t* orow = a.out + (size_t)col_tok[i] * a.out_stride + (size_t)col_head[i] * DH;
+    bf16_t* orow = a.out + (size_t)col_tok[i] * a.out_stride + (size_t)col_head[i] * a.out_pitch + a.out_offset;
     // acc[i][t][r] is channel 16 t + 4 g4 + r: four consecutive channels per output block
 #pragma unroll
     for (int t = 0; t < DT; ++t)
@@ -546,11 +567,19 @@ TL_EXPORT int tl_attn_prefill(const void* q, int q_stride, void* out, int out_st
                               const int32_t* block_table, int bt_stride, const int32_t* tile_row,
                               const int32_t* tile_q0, int n_tiles, int n_q_heads, int n_kv_heads, int head_dim,
                               int page_size, int window, float scale, int key_groups, float softcap, int chunk,
-                              const float* sinks, hipStream_t stream) {
+                              const float* sinks, int keep_first, int n_v_heads, int v_pitch, int v_offset, int out_pitch,
+                              int out_offset, hipStream_t stream) {
   if (head_dim != DH) return variant_fail(TL_ERR_ARG, "attn_prefill: built for head_dim %d, called with %d", DH, head_dim);
   if (n_tiles < 0 || n_q_heads <= 0 || n_kv_heads <= 0 || page_size <= 0 || bt_stride <= 0 || window < 0 || chunk < 0 || softcap < 0)
     return variant_fail(TL_ERR_ARG, "attn_prefill: bad sizes");
   if (n_q_heads % n_kv_heads) return variant_fail(TL_ERR_ARG, "attn_prefill: %d query heads are not a multiple of %d kv heads", n_q_heads, n_kv_heads);
+  if (n_v_heads <= 0) n_v_heads = n_kv_heads;
+  if (v_pitch <= 0) v_pitch = DH;
+  if (out_pitch <= 0) out_pitch = DH;
+  if (keep_first < 0 || n_kv_heads % n_v_heads || v_offset < 0 || v_offset + DH > v_pitch || out_offset < 0 || out_offset + DH > out_pitch
+      || v_pitch % 8 || v_offset % 8 || out_pitch % 4 || out_offset % 4)
+    return variant_fail(TL_ERR_ARG, "attn_prefill: kept keys, value heads or the places of values and outputs do not fit");
+  if (keep_first > 0 && softcap > 0) return variant_fail(TL_ERR_UNSUPPORTED, "attn_prefill: kept first keys together with capped scores are not built");
   const int R = n_q_heads / n_kv_heads;
   if (R > 16) return variant_fail(TL_ERR_UNSUPPORTED, "attn_prefill: %d query heads per kv head exceed 16", R);
   if (n_tiles > 65535) return variant_fail(TL_ERR_UNSUPPORTED, "attn_prefill: %d query tiles exceed a launch's 65535", n_tiles);
@@ -566,6 +595,8 @@ TL_EXPORT int tl_attn_prefill(const void* q, int q_stride, void* out, int out_st
   a.qo_indptr = qo_indptr; a.kv_lens = kv_lens; a.block_table = block_table; a.bt_stride = bt_stride;
   a.tile_row = tile_row; a.tile_q0 = tile_q0;
   a.n_kv_heads = n_kv_heads; a.group = R; a.page_size = page_size; a.window = window;
+  a.keep_first = (window > 0 || chunk > 0) ? keep_first : 0; a.n_v_heads = n_v_heads; a.v_pitch = v_pitch; a.v_offset = v_offset;
+  a.out_pitch = out_pitch; a.out_offset = out_offset;
   a.page_shift = 0;
   while ((1 << a.page_shift) < page_size) ++a.page_shift;
   if ((1 << a.page_shift) != page_size)
@@ -579,16 +610,18 @@ TL_EXPORT int tl_attn_prefill(const void* q, int q_stride, void* out, int out_st
   a.cap_over_scale = softcap > 0 ? softcap / scale : 0.f;
   a.two_scale_over_cap_log2e = softcap > 0 ? 2.0f * scale / softcap * 1.4426950408889634f : 0.f;
   dim3 grid(n_kv_heads, n_tiles);  // consecutive blocks share a query tile: their loads of q overlap
-  const int mode = softcap > 0 ? 2 : (window > 0 || chunk > 0) ? 1 : 0;
+  const int mode = softcap > 0 ? 2 : a.keep_first > 0 ? 3 : (window > 0 || chunk > 0) ? 1 : 0;
   const int threads = kWaves * kWave;
 #define TL_PREFILL_LAUNCH(rp)                                                                      \
   do {                                                                                             \
     if (key_groups == 2) {                                                                         \
       if (mode == 2) attn_prefill_kernel<rp, 2, 2><<<grid, 2 * threads, 0, stream>>>(a);           \
+      else if (mode == 3) attn_prefill_kernel<rp, 3, 2><<<grid, 2 * threads, 0, stream>>>(a);      \
       else if (mode == 1) attn_prefill_kernel<rp, 1, 2><<<grid, 2 * threads, 0, stream>>>(a);      \
       else attn_prefill_kernel<rp, 0, 2><<<grid, 2 * threads, 0, stream>>>(a);                     \
     } else {                                                                                       \
       if (mode == 2) attn_prefill_kernel<rp, 2, 1><<<grid, threads, 0, stream>>>(a);               \
+      else if (mode == 3) attn_prefill_kernel<rp, 3, 1><<<grid, threads, 0, stream>>>(a);          \
       else if (mode == 1) attn_prefill_kernel<rp, 1, 1><<<grid, threads, 0, stream>>>(a);          \
       else attn_prefill_kernel<rp, 0, 1><<<grid, threads, 0, stream>>>(a);                         \
     }                                                                                              \

@@ -164,7 +164,7 @@ def attention_generic_split(
 
 
 _DECODE_SIGNATURES = {
-    "tl_attn_decode": [_P, _I, _P, _I, _P, _P, _P, _P, _P, _I, _I, _I, _I, _I, _I, _I, _F, _I, _I, _P, _P, _F, _I, _P, _P],
+    "tl_attn_decode": [_P, _I, _P, _I, _P, _P, _P, _P, _P, _I, _I, _I, _I, _I, _I, _I, _F, _I, _I, _P, _P, _F, _I, _P, _I, _I, _I, _I, _I, _I, _P],
 }
 DECODE_HEAD_DIMS = (32, 64, 128, 256)
 _DECODE_BLOCK_KEYS = 64  # keys one block pass covers (4 waves x 16): splits are multiples of it
@@ -248,10 +248,18 @@ def attention_decode(
     softcap: float = 0.0,
     chunk: int = 0,
     sinks: Optional[torch.Tensor] = None,
+    keep_first: int = 0,
+    value_heads: Optional[int] = None,
+    v_offset: int = 0,
 ) -> torch.Tensor:
     """Attention of single-token queries over their requests' pages with the split-KV MFMA kernel.
     ``longest``: an upper bound of any token's visible key range, counted from its 16-aligned first
-    visible key (position + 1 without a window).  ``softcap``, ``chunk``, ``sinks``: as ``attention_generic``."""
+    visible key (position + 1 without a window; kept first keys are counted here).  ``softcap``, ``chunk``, ``sinks``: as ``attention_generic``.
+    ``keep_first``: behind a window a query also sees that many first positions of its request.  ``value_heads``,
+    ``v_offset``: the value pages are [pages, value_heads, page, v_pitch] with ``value_heads`` dividing the kv heads
+    (key head g reads value head ``g % value_heads``) and rows of ``v_pitch`` >= dh channels, of which this call takes
+    dh from ``v_offset``; the outputs of a head then lie ``v_pitch`` apart in ``out`` ([n, Hq * v_pitch]), this call's at
+    ``v_offset``: values wider than the keys are worked off in calls of dh channels each."""
     if sinks is not None and (not sinks.is_cuda or sinks.dtype != torch.float32 or sinks.numel() != n_q_heads or not sinks.is_contiguous()):
         raise KernelError(f"attention_decode: sinks must be a contiguous float32 GPU vector of {n_q_heads} entries")
     _gpu(qkv, k_pages, v_pages, token_seq, positions, block_table)
@@ -267,11 +275,20 @@ def attention_decode(
     if block_table.dim() != 2 or block_table.dtype != torch.int32 or block_table.stride(1) != 1:
         raise KernelError("attention_decode: block_table must be an int32 matrix")
     page_size = k_pages.shape[2]
-    for pg in (k_pages, v_pages):
-        if pg.dim() != 4 or pg.shape[1:] != (n_kv_heads, page_size, head_dim) or pg.dtype != qkv.dtype or not pg.is_contiguous():
-            raise KernelError("attention_decode: pages must be contiguous [pages, Hkv, page_size, dh] bfloat16")
+    v_heads = n_kv_heads if value_heads is None else int(value_heads)
+    v_pitch = v_pages.shape[3] if v_pages.dim() == 4 else -1
+    if keep_first < 0 or v_heads <= 0 or n_kv_heads % v_heads or v_offset < 0 or v_offset + head_dim > v_pitch or v_pitch % 8 or v_offset % 8:
+        raise KernelError("attention_decode: kept keys, value heads or the place of the values inside their rows do not fit")
+    if k_pages.dim() != 4 or k_pages.shape[1:] != (n_kv_heads, page_size, head_dim) or k_pages.dtype != qkv.dtype or not k_pages.is_contiguous():
+        raise KernelError("attention_decode: key pages must be contiguous [pages, Hkv, page_size, dh] bfloat16")
+    if v_pages.dim() != 4 or v_pages.shape[:3] != (k_pages.shape[0], v_heads, page_size) or v_pages.dtype != qkv.dtype or not v_pages.is_contiguous():
+        raise KernelError("attention_decode: value pages must be contiguous [pages, value heads, page_size, >= dh] bfloat16")
     if out is None:
-        out = torch.empty((n, n_q_heads * head_dim), dtype=qkv.dtype, device=qkv.device)
+        out = torch.empty((n, n_q_heads * v_pitch), dtype=qkv.dtype, device=qkv.device)
+    elif out.dim() != 2 or out.stride(1) != 1 or out.shape[0] < n or out.shape[1] < n_q_heads * v_pitch or out.dtype != qkv.dtype:
+        raise KernelError("attention_decode: out must be row-major [tokens, >= Hq * value row] bfloat16")
+    if keep_first > 0 and (window > 0 or chunk > 0):
+        longest = longest + (keep_first + 15) // 16 * 16
     if split_size is None:
         split_size, n_splits = plan_decode_splits(n, n_kv_heads, longest, head_dim, uneven=uneven)
     else:
@@ -286,7 +303,8 @@ def attention_decode(
             qkv.data_ptr(), qkv.stride(0), out.data_ptr(), out.stride(0), k_pages.data_ptr(), v_pages.data_ptr(),
             token_seq.data_ptr(), positions.data_ptr(), block_table.data_ptr(), block_table.stride(0), n,
             n_q_heads, n_kv_heads, head_dim, page_size, window, float(scale), split_size, n_splits,
-            _ptr(ws_o), _ptr(ws_ml), float(softcap), int(chunk), _ptr(sinks), _stream(),
+            _ptr(ws_o), _ptr(ws_ml), float(softcap), int(chunk), _ptr(sinks), int(keep_first) if (window > 0 or chunk > 0) else 0, v_heads,
+            v_pitch, int(v_offset), v_pitch, int(v_offset), _stream(),
         ),
         lib,
         "tl_variant_last_error",
@@ -296,7 +314,7 @@ def attention_decode(
 
 # ----------------------------------------------------------------------------- prefill attention (bfloat16, MFMA)
 _PREFILL_SIGNATURES = {
-    "tl_attn_prefill": [_P, _I, _P, _I, _P, _P, _P, _P, _P, _I, _P, _P, _I, _I, _I, _I, _I, _I, _F, _I, _F, _I, _P, _P],
+    "tl_attn_prefill": [_P, _I, _P, _I, _P, _P, _P, _P, _P, _I, _P, _P, _I, _I, _I, _I, _I, _I, _F, _I, _F, _I, _P, _I, _I, _I, _I, _I, _I, _P],
 }
 PREFILL_HEAD_DIMS = (32, 64, 128, 256)
 
@@ -394,10 +412,18 @@ def attention_prefill(
     softcap: float = 0.0,
     chunk: int = 0,
     sinks: Optional[torch.Tensor] = None,
+    keep_first: int = 0,
+    value_heads: Optional[int] = None,
+    v_offset: int = 0,
 ) -> torch.Tensor:
     """Causal attention of the rows named by the tile lists (see ``prefill_tiles``) with the MFMA
     prefill kernel.  Token t of ``qkv`` / ``out`` is token t of ``qo_indptr``'s numbering.
-    ``key_groups`` = 2: two sets of waves per block share a tile's keys between them."""
+    ``key_groups`` = 2: two sets of waves per block share a tile's keys between them.
+    ``keep_first``: behind a window a query also sees that many first positions of its request.  ``value_heads``,
+    ``v_offset``: the value pages are [pages, value_heads, page, v_pitch] with ``value_heads`` dividing the kv heads
+    (key head g reads value head ``g % value_heads``) and rows of ``v_pitch`` >= dh channels, of which this call takes
+    dh from ``v_offset``; the outputs of a head then lie ``v_pitch`` apart in ``out`` ([n, Hq * v_pitch]), this call's at
+    ``v_offset``: values wider than the keys are worked off in calls of dh channels each."""
     _gpu(qkv, k_pages, v_pages, qo_indptr, kv_lens, block_table, tile_row, tile_q0, out)
     for t, what in ((qo_indptr, "qo_indptr"), (kv_lens, "kv_lens"), (tile_row, "tile_row"), (tile_q0, "tile_q0")):
         _i32(t, what)
@@ -405,8 +431,6 @@ def attention_prefill(
         raise KernelError("attention_prefill takes bfloat16")
     if qkv.dim() != 2 or qkv.stride(1) != 1 or qkv.shape[1] < n_q_heads * head_dim:
         raise KernelError("attention_prefill: qkv must be row-major with at least Hq * dh columns")
-    if out.dim() != 2 or out.stride(1) != 1 or out.shape[0] != qkv.shape[0] or out.shape[1] < n_q_heads * head_dim:
-        raise KernelError("attention_prefill: out must be row-major [tokens, >= Hq * dh]")
     if tile_row.numel() != tile_q0.numel():
         raise KernelError("attention_prefill: tile lists differ in length")
     if block_table.dim() != 2 or block_table.dtype != torch.int32 or block_table.stride(1) != 1:
@@ -414,16 +438,24 @@ def attention_prefill(
     if kv_lens.numel() != block_table.shape[0] or qo_indptr.numel() != kv_lens.numel() + 1:
         raise KernelError("attention_prefill: qo_indptr, kv_lens and block_table disagree about the rows")
     page_size = k_pages.shape[2]
-    for pg in (k_pages, v_pages):
-        if pg.dim() != 4 or pg.shape[1:] != (n_kv_heads, page_size, head_dim) or pg.dtype != qkv.dtype or not pg.is_contiguous():
-            raise KernelError("attention_prefill: pages must be contiguous [pages, Hkv, page_size, dh] bfloat16")
+    v_heads = n_kv_heads if value_heads is None else int(value_heads)
+    v_pitch = v_pages.shape[3] if v_pages.dim() == 4 else -1
+    if keep_first < 0 or v_heads <= 0 or n_kv_heads % v_heads or v_offset < 0 or v_offset + head_dim > v_pitch or v_pitch % 8 or v_offset % 8:
+        raise KernelError("attention_prefill: kept keys, value heads or the place of the values inside their rows do not fit")
+    if k_pages.dim() != 4 or k_pages.shape[1:] != (n_kv_heads, page_size, head_dim) or k_pages.dtype != qkv.dtype or not k_pages.is_contiguous():
+        raise KernelError("attention_prefill: key pages must be contiguous [pages, Hkv, page_size, dh] bfloat16")
+    if v_pages.dim() != 4 or v_pages.shape[:3] != (k_pages.shape[0], v_heads, page_size) or v_pages.dtype != qkv.dtype or not v_pages.is_contiguous():
+        raise KernelError("attention_prefill: value pages must be contiguous [pages, value heads, page_size, >= dh] bfloat16")
+    if out.dim() != 2 or out.stride(1) != 1 or out.shape[0] != qkv.shape[0] or out.shape[1] < n_q_heads * v_pitch:
+        raise KernelError("attention_prefill: out must be row-major [tokens, >= Hq * value row]")
     lib = variant("attn_prefill", head_dim, _PREFILL_SIGNATURES)
     check(
         lib.tl_attn_prefill(
             qkv.data_ptr(), qkv.stride(0), out.data_ptr(), out.stride(0), k_pages.data_ptr(), v_pages.data_ptr(),
             qo_indptr.data_ptr(), kv_lens.data_ptr(), block_table.data_ptr(), block_table.stride(0),
             tile_row.data_ptr(), tile_q0.data_ptr(), tile_row.numel(), n_q_heads, n_kv_heads, head_dim, page_size,
-            window, float(scale), int(key_groups), float(softcap), int(chunk), _ptr(sinks), _stream(),
+            window, float(scale), int(key_groups), float(softcap), int(chunk), _ptr(sinks), int(keep_first), v_heads, v_pitch, int(v_offset),
+            v_pitch, int(v_offset), _stream(),
         ),
         lib,
         "tl_variant_last_error",
