@@ -644,6 +644,50 @@ def test_trace_replay_program(tmp_path):
             assert distance(row, truth[rid][pos], scale) < FP32_TOL, (s["step"], rid, pos)
 
 
+ODD = {
+    "width_50": models.model(33, 50, 3, 1.5, 1e-5, [
+        models.layer("attention", models.diff_attention(3, 1, 10, 6, 0.3, 0.5, _R(6, 100.0), 9, keep_first=2, conv=2), models.moe(14, 3, 2, 1.5, shared=10)),
+        models.layer("parallel", models.pair(models.left(2, 1, 12, 10, 0.3, _R(4, 100.0), 7, keep_first=1), models.right(2, 6, 10, 3.0, 2), 0.8, 0.7), None),
+        models.layer("latent_attention", models.latent(3, 6, 2, 10, 14, 0.3, 11), models.moe(9, 2, 1, 1.0, groups=(2, 1))),
+        models.layer("attention", models.diff_attention(1, 1, 10, 6, 0.3, 0.2, _R(6, 100.0), 30, keep_first=0, kv_from=0), None),
+    ]),
+    "width_52": models.model(70, 52, 5, 1.0, 1e-5, [
+        models.layer("latent_attention", models.latent(1, 4, 4, 4, 12, 0.4, 1000), models.moe(12, 4, 2, 2.0, groups=(2, 2), shared=20)),
+        models.layer("attention", models.diff_attention(2, 2, 4, 12, 0.4, 0.9, _R(4, 10.0), 5, keep_first=5, conv=3), None),
+    ]),
+}
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+@pytest.mark.parametrize("name", sorted(ODD))
+def test_widths_that_are_no_multiple_of_eight(tmp_path, name, dtype):
+    """Rows that no 16-byte load fits, heads of a handful of channels, more streams than usual: the kernels' plain forms."""
+    from torchllms_amd.engine import Engine, StepEntry
+
+    folder = folder_for(dtype, tmp_path / name, ODD[name], seed=2)
+    cfg, weights = models.read_folder(folder)
+    tokens = random_tokens(90, cfg["vocab"], 4)
+    truth, scale = truth_of(cfg, weights, {"r": tokens})
+    engine = Engine.from_folder(folder, dtype=dtype, page_size=4, num_pages=60, max_seqs=2)
+    engine.admit("whole")
+    whole = engine.step([StepEntry("whole", tokens, list(range(90)))]).cpu()
+    engine.admit("cut")
+    rows, at = [], 0
+    for n in (3, 2, 40, 1, 1, 35, 1, 1, 1, 5):
+        rows.append(engine.step([StepEntry("cut", tokens[at : at + n], list(range(n)))]).cpu())
+        at += n
+    assert at == 90
+    cut = torch.cat(rows)
+    for what, got in (("whole", whole), ("cut", cut)):
+        dists = [distance(got[i], truth["r"][i], scale) for i in range(90)]
+        if dtype == "float32":
+            assert max(dists) < FP32_TOL, f"{name}/{what}: {max(dists)}"
+        else:
+            assert_within_rounding(dists, 2 * BF16_TOL, f"{name}/{what}")
+    if dtype == "float32":
+        assert torch.equal(whole, cut)
+
+
 # ----------------------------------------------------------------------------- random configurations
 def random_config(seed: int) -> dict:
     """A Nosuzen configuration drawn from a seed: every size, constant and the order of layers."""
