@@ -339,7 +339,7 @@ def test_matrix_core_attention_with_kept_first_keys_and_wide_values(Hq, Hk, Hv, 
             assert float(err.max()) < 3e-2 * max(1.0, float(want.abs().max())), (first, count, groups, int(err.argmax()) + first, float(err.max()))
 
 
-@pytest.mark.parametrize("S,D,n", [(3, 256, 70), (1, 64, 5), (4, 50, 33), (8, 36, 2)])
+@pytest.mark.parametrize("S,D,n", [(3, 256, 70), (1, 64, 5), (4, 50, 33), (8, 36, 2), (16, 128, 9), (11, 30, 40)])
 def test_streams_kernel_against_the_formulas(S, D, n):
     from torchllms_amd.kernels import ops
 
@@ -612,6 +612,37 @@ def test_a_preempted_request_starts_again_from_clean_state(tmp_path):
     assert tight.last_stats["preemptions"] > 0
     assert [r.token_ids for r in got] == [r.token_ids for r in want]
     tight.engine.cache.check_invariants()
+
+
+def test_generate_command_line_with_random_weights(tmp_path):
+    """The generate program given nothing but a config.json: ``--random-weights --seed`` draws the weights that
+    ``write_model_folder`` would write for that seed, so the plain model can say which tokens to expect."""
+    import json
+    import subprocess
+    import sys
+    from pathlib import Path
+
+    from torchllms_amd.config.nosuzen import NosuzenConfig
+    from torchllms_amd.weights import write_model_folder
+
+    root = Path(__file__).resolve().parent.parent
+    folder = tmp_path / "only_config"
+    folder.mkdir()
+    (folder / "config.json").write_text(json.dumps(models.CONFIG_B))
+    prompt = random_tokens(13, models.CONFIG_B["vocab"], 21)
+    proc = subprocess.run(
+        [sys.executable, "-m", "torchllms_amd.inference.generate", "--model", str(folder), "--dtype", "float32", "--random-weights",
+         "--seed", "7", "--max-new-tokens", "6", "--prompt-ids", *map(str, prompt)],
+        capture_output=True, text=True, cwd=root, timeout=300,
+    )
+    assert proc.returncode == 0, proc.stderr[-2000:]
+    got = [int(t) for t in proc.stdout.split()[-6:]]
+    written = write_model_folder(tmp_path / "written", NosuzenConfig.from_dict(models.CONFIG_B), seed=7, dtype=torch.float32)
+    cfg, weights = models.read_folder(written)
+    toks = list(prompt)
+    for _ in range(6):
+        toks.append(int(plain.forward(cfg, weights, toks)[-1].argmax()))
+    assert got == toks[len(prompt):]
 
 
 def test_trace_replay_program(tmp_path):

@@ -9,7 +9,7 @@
 
 namespace {
 
-constexpr int kMaxStreams = 8;
+constexpr int kMaxStreams = 16;  // (the weights of all pairs are one entry a thread of a block)
 
 struct StreamWeights {
   float mix[kMaxStreams][kMaxStreams];  // [from][to]

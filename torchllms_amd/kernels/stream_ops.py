@@ -10,7 +10,7 @@ import torch
 from .base import F32, KernelError, _gpu, _i32, _ptr, _stream, check, core, dtype_code
 
 #: the most residual streams the kernels take
-MAX_STREAMS = 8
+MAX_STREAMS = 16
 
 
 def _f32(v: Optional[torch.Tensor], shape, what: str) -> None:
