@@ -19,7 +19,8 @@ struct StreamWeights {
 
 // One thread an element (V of them side by side).  branch (BT) given: the planes are updated in place.  w given: the
 // normed read goes to rows (T); with `gather` the tokens read are gather[0 .. n) (no update then).
-template <typename T, typename BT, int V>
+// MAXS: the most streams this instantiation holds in registers (4, 8 or 16: few streams leave room for many waves).
+template <typename T, typename BT, int V, int MAXS>
 __global__ void __launch_bounds__(256)
 streams_update_kernel(float* __restrict__ x, int S, long long plane, int n, int D, const BT* __restrict__ branch,
                       const float* __restrict__ mix, const float* __restrict__ out_w, const float* __restrict__ in_w,
@@ -42,9 +43,9 @@ streams_update_kernel(float* __restrict__ x, int S, long long plane, int n, int 
   for (long long i = (long long)blockIdx.x * blockDim.x + threadIdx.x; i < total; i += (long long)gridDim.x * blockDim.x) {
     const int t_out = (int)(i / per_row), d0 = (int)(i % per_row) * V;
     const int t = gather ? gather[t_out] : t_out;
-    float xs[kMaxStreams][V];
+    float xs[MAXS][V];
 #pragma unroll
-    for (int s = 0; s < kMaxStreams; ++s)
+    for (int s = 0; s < MAXS; ++s)
       if (s < S) {
         const float* p = x + s * plane + (long long)t * D + d0;
         if constexpr (V == 4) {
@@ -59,21 +60,21 @@ streams_update_kernel(float* __restrict__ x, int S, long long plane, int n, int 
       float y[V];
 #pragma unroll
       for (int e = 0; e < V; ++e) y[e] = to_f32(branch[(long long)t * D + d0 + e]);
-      float nx[kMaxStreams][V];
+      float nx[MAXS][V];
 #pragma unroll
-      for (int r = 0; r < kMaxStreams; ++r)
+      for (int r = 0; r < MAXS; ++r)
         if (r < S) {
 #pragma unroll
           for (int e = 0; e < V; ++e) {
             float acc = 0.f;
 #pragma unroll
-            for (int s = 0; s < kMaxStreams; ++s)
+            for (int s = 0; s < MAXS; ++s)
               if (s < S) acc += sw.mix[s][r] * xs[s][e];
             nx[r][e] = acc + sw.out[r] * y[e];
           }
         }
 #pragma unroll
-      for (int r = 0; r < kMaxStreams; ++r)
+      for (int r = 0; r < MAXS; ++r)
         if (r < S) {
           float* p = x + r * plane + (long long)t * D + d0;
 #pragma unroll
@@ -90,7 +91,7 @@ streams_update_kernel(float* __restrict__ x, int S, long long plane, int n, int 
       for (int e = 0; e < V; ++e) {
         float u = 0.f;
 #pragma unroll
-        for (int s = 0; s < kMaxStreams; ++s)
+        for (int s = 0; s < MAXS; ++s)
           if (s < S) u += sw.in[s] * xs[s][e];
         rows[(long long)t_out * D + d0 + e] = from_f32<T>(tanhf(a * u) * w[d0 + e] + b[d0 + e]);
       }
@@ -155,14 +156,16 @@ TL_EXPORT int tl_streams_update(float* x, int S, long long plane, int n, int D, 
   if (branch && branch_dtype != TL_F32 && branch_dtype != dtype) return tl_fail(TL_ERR_ARG, "streams_update: the branch is 32-bit or of the rows' dtype");
   const bool vec = D % 4 == 0 && ((uintptr_t)x % 16) == 0 && plane % 4 == 0;
   const int blocks = grid_for((long long)n * (vec ? D / 4 : D));
-#define TL_SU(T, BT, V) \
-  streams_update_kernel<T, BT, V><<<blocks, 256, 0, stream>>>(x, S, plane, n, D, (const BT*)branch, mix, out_w, in_w, alpha, w, b, gather, (T*)rows)
+#define TL_SU_M(T, BT, V, M) \
+  streams_update_kernel<T, BT, V, M><<<blocks, 256, 0, stream>>>(x, S, plane, n, D, (const BT*)branch, mix, out_w, in_w, alpha, w, b, gather, (T*)rows)
+#define TL_SU(T, BT, V) do { if (S <= 4) TL_SU_M(T, BT, V, 4); else if (S <= 8) TL_SU_M(T, BT, V, 8); else TL_SU_M(T, BT, V, 16); } while (0)
 #define TL_SU_V(T, BT) do { if (vec) TL_SU(T, BT, 4); else TL_SU(T, BT, 1); } while (0)
   if (dtype == TL_F32) TL_SU_V(float, float);
   else if (branch && branch_dtype == TL_F32) TL_SU_V(bf16_t, float);
   else TL_SU_V(bf16_t, bf16_t);
 #undef TL_SU_V
 #undef TL_SU
+#undef TL_SU_M
   return tl_check_launch("streams_update");
 }
 
