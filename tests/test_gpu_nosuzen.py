@@ -145,6 +145,8 @@ ALONE = {
     "differential_no_conv_no_window_edge": models.layer("attention", models.diff_attention(2, 2, 16, 16, 0.3, 0.1, _R(16, 100.0), 1000)),
     "differential_one_tap_odd_sizes": models.layer("attention", models.diff_attention(3, 1, 20, 36, 0.2, 0.8, _R(0), 19, keep_first=19, conv=1)),
     "differential_wide": models.layer("attention", models.diff_attention(2, 1, 128, 256, 0.08, 0.6, _R(64, 1e6, (4.0, 64, 16.0, 1.0)), 64, keep_first=70, conv=2)),
+    "differential_matrix_cores": models.layer("attention", models.diff_attention(4, 2, 64, 128, 0.12, 0.5, _R(64, 1e4, (4.0, 64, 16.0, 1.0)), 50, keep_first=7, conv=2)),
+    "differential_matrix_cores_same_width": models.layer("attention", models.diff_attention(2, 1, 128, 128, 0.09, 0.3, _R(32, 1e4), 33, keep_first=40)),
     "latent_matrix_cores": models.layer("latent_attention", models.latent(4, 32, 32, 32, 96, 0.15, 40, scaling=(2.0, 64, 32.0, 1.0))),
     "latent_odd": models.layer("latent_attention", models.latent(3, 20, 6, 28, 50, 0.2, 25, base=50.0)),
     "latent_nothing_rotated_wide_latent": models.layer("latent_attention", models.latent(2, 16, 0, 8, 288, 0.2, 90)),
@@ -478,10 +480,11 @@ def test_long_prompts_with_sharp_attention_and_long_memory(tmp_path, dtype):
     from torchllms_amd.engine import Engine, StepEntry
 
     cfg_dict = models.model(97, 64, 3, 2.0, 1e-5, [
-        models.layer("attention", models.diff_attention(2, 1, 32, 48, 0.2, 0.5, _R(32, 1e5), 300, keep_first=17, conv=3), models.moe(32, 4, 2, 2.0, groups=(2, 1), shared=16)),
+        # (heads of 32 channels with values twice as wide: in bfloat16 the matrix-core kernels run them, the reader below too)
+        models.layer("attention", models.diff_attention(2, 1, 32, 64, 0.2, 0.5, _R(32, 1e5), 300, keep_first=17, conv=3), models.moe(32, 4, 2, 2.0, groups=(2, 1), shared=16)),
         models.layer("parallel", models.pair(models.left(4, 2, 32, 32, 0.2, _R(16, 1e4, (4.0, 128, 16.0, 1.0)), 130, keep_first=40),
                                              models.right(2, 32, 32, 64.0, 8), 1.0, 0.6), None),
-        models.layer("attention", models.diff_attention(2, 1, 32, 48, 0.2, 0.3, _R(32, 1e5), 129, keep_first=33, conv=2, kv_from=0), None),
+        models.layer("attention", models.diff_attention(4, 1, 32, 64, 0.2, 0.3, _R(32, 1e5), 129, keep_first=33, conv=2, kv_from=0), None),
         models.layer("latent_attention", models.latent(2, 32, 16, 32, 48, 0.15, 257, scaling=(2.0, 256, 32.0, 1.0)), models.moe(24, 3, 1, 1.0)),
     ])
     folder = folder_for(dtype, tmp_path / "m", cfg_dict, seed=3, sharpen=4.0)
@@ -515,7 +518,7 @@ def test_long_prompts_with_sharp_attention_and_long_memory(tmp_path, dtype):
         assert torch.equal(whole, cut)
     # dropping what lies far back would be seen: the truth of the last 100 tokens alone is another
     short = plain.forward(cfg, weights, tokens[600:])
-    assert max(distance(short[i], truth["r"][600 + i], scale) for i in range(50, 100)) > 5 * tol
+    assert max(distance(short[i], truth["r"][600 + i], scale) for i in range(50, 100)) > 3 * tol
 
 
 def test_a_slot_that_is_used_again_starts_from_zero(tmp_path):
