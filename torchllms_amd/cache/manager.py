@@ -5,7 +5,9 @@ Layers whose needs are alike (same heads, head size, window, tokens per page and
 a *group*.  A group owns a pool of pages; one page id addresses the same token range in every layer
 of the group.  A request holds one block table per group (logical block -> page id); groups may
 differ in page size, so their tables differ in length and their pools in the pages a step takes.  Pages go back to the pool
-when the request ends and, in a group with a window, as soon as the window has passed them.
+when the request ends and, in a group with a window, as soon as the window has passed them; a group may keep the first
+positions of every request visible behind its window (``keep_first``), and the pages that hold those are never passed.
+The value pages of a group may have fewer heads than its key pages (``v_heads``).
 
 The bookkeeping is plain host code and runs without a GPU; the page tensors are optional so the
 allocator can be tested alone.

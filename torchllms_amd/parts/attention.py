@@ -408,7 +408,12 @@ class DifferentialAttention(Mixer):
 
     def bind(self, tensors: Dict[str, torch.Tensor]) -> None:
         parts = [("q", self.H)] if self.shares_kv else [("q", self.H), ("k", self.G), ("v", 0)]
-        ordered = lambda name, heads, suffix="": (self._maps_first(tensors[name + suffix], heads) if heads else tensors[name + suffix])  # noqa: E731
+
+        def ordered(name, heads, suffix=""):
+            """Rows of q and k with the maps first; the values' rows as they are (heads 0)."""
+            t = tensors[name + suffix]
+            return self._maps_first(t, heads) if heads else t
+
         self.wqkv = torch.cat([ordered(n, h) for n, h in parts], dim=0).contiguous()
         if self.taps > 0:
             self.conv_w = torch.cat([ordered(n, h, ".conv") for n, h in parts], dim=0).float().t().contiguous()  # [taps, channels]
