@@ -372,15 +372,15 @@ def nosuzen_config(shape: dict, n_layers: int) -> dict:
     stay, a token uses two, beside a shared expert of a quarter of that width."""
     D, H, G, dh, ff = shape["hidden_size"], shape["num_attention_heads"], shape["num_key_value_heads"], shape["head_dim"], shape["intermediate_size"]
     yarn = {"factor": 8.0, "original": 8192, "fast": 32.0, "slow": 1.0}
-    differential = {"heads": max(H // 2, 1), "kv_heads": max(G // 2, 1), "dim": dh, "vdim": 2 * dh, "scale": dh ** -0.5, "diff": 0.6, "conv": 4,
+    differential = {"heads": max(H // 2, 1), "kv_heads": max(G // 2, 1), "dim": dh, "vdim": 2 * dh, "scale": dh ** -0.5, "diff": 0.5, "conv": 4,
                     "rot": {"dims": dh, "base": shape["rope_theta"]}, "mask": {"size": 4096, "keep_first": 64}}
     pair = {"left": {"heads": H, "kv_heads": G, "dim": dh, "vdim": dh, "scale": dh ** -0.5, "rot": {"dims": dh // 2, "base": shape["rope_theta"], "scaling": yarn},
                      "mask": {"size": 4096, "keep_first": 64}},
-            "right": {"heads": max(H // 2, 1), "dim": dh, "vdim": dh, "tau": 16.0, "decay_rank": 64},
+            "right": {"heads": max(H // 2, 1), "dim": dh, "vdim": dh, "tau": 8.0, "decay_rank": 64},
             "left_scale": 0.6, "right_scale": 0.5}
     through_latent = {"heads": H, "dim": dh, "rot_dim": 64, "vdim": dh, "kv_rank": 192, "scale": (dh + 64) ** -0.5,
                       "rot": {"dims": 64, "base": 10000.0, "scaling": yarn}, "mask": {"size": 4096}}
-    moe = {"kind": "moe", "expert": {"ff": ff // 4}, "router": {"experts": 8, "top": 2, "scale": 2.0, "groups": {"count": 4, "keep": 2}}, "shared": {"ff": ff // 4}}
+    moe = {"kind": "moe", "expert": {"ff": ff // 4}, "router": {"experts": 8, "top": 2, "scale": 1.5, "groups": {"count": 4, "keep": 2}}, "shared": {"ff": ff // 4}}
     layers = []
     for i in range(n_layers):
         kind = i % 4

@@ -87,10 +87,10 @@ CONFIG_B = model(77, 96, 1, 1.0, 1e-6, [
     layer("latent_attention", latent(3, 24, 16, 20, 112, 0.15, 64, base=300.0), moe(16, 3, 2, 1.0)),
 ])
 CONFIG_C = model(200, 128, 4, 6.0, 1e-5, [
-    layer("latent_attention", latent(4, 32, 32, 32, 96, 0.125, 50, scaling=(2.0, 64, 32.0, 1.0)), moe(56, 8, 3, 2.0, groups=(2, 1), shared=72)),
-    layer("attention", diff_attention(2, 1, 48, 96, 0.14, 0.6, rot(48, 1e6), 36, keep_first=8, conv=3), moe(32, 5, 2, 0.5)),
+    layer("latent_attention", latent(4, 40, 32, 24, 224, 0.11, 50, scaling=(4.0, 64, 16.0, 2.0)), moe(56, 10, 3, 1.75, groups=(2, 1), shared=72)),
+    layer("attention", diff_attention(2, 1, 40, 80, 0.16, 0.35, rot(40, 5e5), 36, keep_first=8, conv=3), moe(32, 5, 2, 0.5)),
     layer("parallel", pair(left(2, 1, 128, 128, 0.09, rot(64, 1000.0), 28, keep_first=9), right(4, 64, 32, 4.0, 16), 0.8, 0.2), moe(32, 7, 2, 1.0, shared=8)),
-    layer("attention", diff_attention(4, 1, 48, 96, 0.14, 0.2, rot(0, 1e4), 60, keep_first=2, conv=5, kv_from=1), None),
+    layer("attention", diff_attention(4, 1, 40, 80, 0.16, 0.2, rot(0, 1e4), 60, keep_first=2, conv=5, kv_from=1), None),
     layer("parallel", pair(left(4, 4, 16, 8, 0.3, rot(0, 100.0), 100, keep_first=0), right(1, 128, 128, 32.0, 3), 0.3, 0.9), moe(24, 2, 2, 3.0, groups=(2, 2))),
 ])
 CONFIGS = {"A": CONFIG_A, "B": CONFIG_B, "C": CONFIG_C}
@@ -129,11 +129,16 @@ def make_folder(path, cfg_dict: dict, seed: int = 0, dtype=torch.bfloat16, sharp
         elif leaf in ("norm1.b", "norm2.b", "final.norm.b"):
             t = 0.3 * torch.randn(t.shape, generator=gen)
         elif last == "alpha":
-            t = 0.5 + 2.0 * torch.rand(t.shape, generator=gen)
-        elif leaf.startswith("hc") and last in ("in", "out"):
+            # (a steep tanh over a sum of several streams acts like a sign: channels near zero would turn rounding into
+            # whole steps, in the plain model as in the engine; steepness and read weights shrink with the streams)
+            t = (0.5 + 2.0 * torch.rand(t.shape, generator=gen)) / cfg_dict["streams"]
+        elif leaf.startswith("hc") and last == "in":
+            t = (0.4 + 0.8 * torch.rand(t.shape, generator=gen)) / cfg_dict["streams"]
+        elif leaf.startswith("hc") and last == "out":
             t = 0.4 + 0.8 * torch.rand(t.shape, generator=gen)
         elif leaf.startswith("hc") and last == "mix":
-            t = torch.eye(t.shape[0]) * 0.8 + 0.3 * torch.randn(t.shape, generator=gen)
+            # (well inside what keeps the streams from growing layer after layer: rounding would grow with them)
+            t = torch.eye(t.shape[0]) * 0.6 + (0.3 / t.shape[0]) * torch.randn(t.shape, generator=gen)
         elif last == "norm":
             t = 1.0 + 0.2 * torch.randn(t.shape, generator=gen)
         elif last in ("lq1", "lk1", "lq2", "lk2"):
